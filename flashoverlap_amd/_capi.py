@@ -1,0 +1,118 @@
+"""ctypes binding of libfo_kernels.so (the C ABI declared in include/flashoverlap.h).
+
+There is no CPU fallback: if the library has not been built, loading raises.
+"""
+import ctypes
+import os
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+KERNEL_LIB = os.path.join(_PKG, "lib", "libfo_kernels.so")
+SHIM_LIB = os.path.join(_PKG, "lib", "libst_pybinding.so")
+
+F16, BF16 = 0, 1
+
+c_int, c_i64, c_f32, vp = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
+
+# name -> (restype, argtypes); one entry per symbol of include/flashoverlap.h
+SIGNATURES = {
+    "fo_error_string": (ctypes.c_char_p, [c_int]),
+    "fo_version": (c_int, []),
+    "fo_algo_count": (c_int, []),
+    "fo_algo_info": (c_int, [c_int, vp]),
+    "fo_schedule_order": (c_int, [c_int, c_int, c_int, vp]),
+    "fo_gemm": (c_int, [c_int, c_int, c_int, c_int, vp, vp, vp, c_int, vp]),
+    "fo_gemm_signal": (c_int, [c_int, c_int, c_int, c_int, c_int, vp, c_int, vp, vp, vp, vp, vp,
+                               c_int, c_int, vp]),
+    "fo_gemm_scatter": (c_int, [c_int, c_int, c_int, c_int, c_int, vp, c_int, vp, vp, vp, vp, vp, vp,
+                                c_int, c_int, vp]),
+    "fo_wait": (c_int, [c_int, vp, vp]),
+    "fo_wait_bounded": (c_int, [c_int, vp, c_i64, vp, vp]),
+    "fo_consumer_reduce": (c_int, [c_int, vp, vp, c_i64, vp]),
+    "fo_consumer_reduce_rs": (c_int, [c_int, vp, vp, c_i64, c_int, c_i64, vp]),
+    "fo_wait_reduce_groups": (c_int, [c_int, vp, vp, vp, vp, c_int, c_i64, c_int, c_i64, vp, c_int,
+                                      vp]),
+    "fo_reorder_rmsnorm": (c_int, [c_int, vp, vp, vp, c_int, c_int, c_int, c_int, c_int, vp, c_f32,
+                                   vp]),
+    "fo_rmsnorm": (c_int, [c_int, vp, vp, vp, c_int, c_int, c_f32, vp]),
+    "fo_overlap_create": (c_int, [ctypes.POINTER(vp)]),
+    "fo_overlap_destroy": (c_int, [vp]),
+    "fo_overlap_set_gemm_stream": (c_int, [vp, vp]),
+    "fo_overlap_init": (c_int, [vp]),
+    "fo_overlap_set_world": (c_int, [vp, c_int, c_int]),
+    "fo_overlap_set_accumulator": (c_int, [vp, vp, c_i64]),
+    "fo_overlap_set_fused_consumer": (c_int, [vp, c_int]),
+    "fo_overlap_comm_stream": (vp, [vp]),
+    "fo_overlap_gemm": (c_int, [vp, c_int, c_int, c_int, c_int, vp, vp, vp, c_int]),
+    "fo_overlap_gemm_allreduce": (c_int, [vp, c_int, c_int, c_int, c_int, vp, vp, vp, vp, vp, c_int,
+                                          c_int, c_int, vp, vp, c_int, c_int, c_int]),
+    "fo_overlap_gemm_reducescatter": (c_int, [vp, c_int, c_int, c_int, c_int, vp, vp, vp, vp, vp, vp,
+                                              vp, c_int, c_int, c_int, vp, vp, c_int, c_int, c_int]),
+    "fo_overlap_gemm_allreduce_serial": (c_int, [vp, c_int, c_int, c_int, c_int, vp, vp, vp, c_int]),
+    "fo_overlap_seg_allreduce": (c_int, [vp, c_int, vp, c_i64, vp, c_int, c_int]),
+}
+
+_lib = None
+
+
+class FlashOverlapError(RuntimeError):
+    def __init__(self, what, code):
+        self.code = code
+        msg = lib().fo_error_string(code).decode() if _lib is not None else "?"
+        super().__init__(f"{what} failed: {msg} (code {code})")
+
+
+def lib():
+    """Load libfo_kernels.so once and attach the prototypes."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(KERNEL_LIB):
+            raise ImportError(
+                f"{KERNEL_LIB} is missing: build it with `python -m flashoverlap_amd.build` "
+                "(hipcc, gfx950). There is no CPU fallback.")
+        L = ctypes.CDLL(KERNEL_LIB)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(L, name)  # AttributeError if the library does not export it
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def check(code, what):
+    if code != 0:
+        raise FlashOverlapError(what, code)
+
+
+def algo_table():
+    """The 102 x 12 Algo table as a list of tuples."""
+    L = lib()
+    out = []
+    buf = (ctypes.c_int32 * 12)()
+    for a in range(L.fo_algo_count()):
+        check(L.fo_algo_info(a, buf), "fo_algo_info")
+        out.append(tuple(buf))
+    return out
+
+
+def algo_tile(algo):
+    buf = (ctypes.c_int32 * 12)()
+    check(lib().fo_algo_info(int(algo), buf), "fo_algo_info")
+    return buf[0], buf[1]
+
+
+def find_algo(bm, bn, swizzle=None, tbk=None, stages=None):
+    """First Algo index whose (TbM, TbN[, Swizzle, TbK, Stages]) match."""
+    for i, row in enumerate(algo_table()):
+        if row[0] == bm and row[1] == bn and (swizzle is None or row[10] == swizzle) and (
+                tbk is None or row[2] == tbk) and (stages is None or row[9] == stages):
+            return i
+    raise ValueError(f"no Algo with tile {bm}x{bn} swizzle={swizzle}")
+
+
+def schedule_order(algo, M, N):
+    """Tile ids in workgroup dispatch order (the analytic hint)."""
+    bm, bn = algo_tile(algo)
+    T = (M // bm) * (N // bn)
+    buf = (ctypes.c_int32 * T)()
+    check(lib().fo_schedule_order(int(algo), M, N, buf), "fo_schedule_order")
+    return list(buf)

@@ -1,0 +1,104 @@
+// Algo index space, raster choice and the analytic tile issue order.
+#include <mutex>
+
+#include "fo_common.h"
+
+namespace {
+
+fo_algo_entry g_table[128];
+int g_count = 0;
+std::once_flag g_once;
+
+// Same enumeration rule as the reference generator (tool/generate_instances.py:5-37):
+// nested product with TbM slowest and Swizzle fastest, minus the shapes CUTLASS
+// could not instantiate; the index is the position among the survivors.
+void build_table() {
+    const int tb[] = {128, 256}, tk[] = {32, 64}, stages[] = {3, 4, 5};
+    const int swz[] = {1, 2, 3, 4, 6, 8};
+    int n = 0;
+    for (int tbm : tb)
+        for (int tbn : tb)
+            for (int tbk : tk)
+                for (int wk : tk)
+                    for (int st : stages)
+                        for (int sw : swz) {
+                            const bool wide = (tbm == 128 && tbn == 256) || (tbm == 256 && tbn == 128);
+                            if (tbm == 256 && tbn == 256) continue;
+                            if (wide && tbk == 64 && (wk == 32 || st >= 4)) continue;
+                            if (tbk % wk) continue;
+                            const int32_t row[12] = {tbm, tbn, tbk, 64, 64, wk, 16, 8, 16, st, sw, 1};
+                            for (int i = 0; i < 12; i++) g_table[n].f[i] = row[i];
+                            n++;
+                        }
+    g_count = n;
+}
+
+}  // namespace
+
+const fo_algo_entry *fo_algo_lookup(int algo) {
+    std::call_once(g_once, build_table);
+    if (algo < 0 || algo >= g_count) return nullptr;
+    return &g_table[algo];
+}
+
+int fo_pick_raster(int algo, int M, int N, fo_raster *r) {
+    const fo_algo_entry *e = fo_algo_lookup(algo);
+    if (!e) return FO_ERR_ALGO;
+    const int bm = e->f[0], bn = e->f[1];
+    if (M <= 0 || N <= 0) return FO_ERR_ARG;
+    if (M % bm || N % bn) return FO_ERR_SHAPE;
+    r->mtm = bm;
+    r->mtn = bn;
+    r->grid_m = M / r->mtm;
+    r->grid_n = N / r->mtn;
+    r->panel = e->f[10] < r->grid_m ? e->f[10] : r->grid_m;
+    r->xcd_remap = ((r->grid_m * r->grid_n) % 8 == 0) ? 1 : 0;
+    return FO_OK;
+}
+
+extern "C" int fo_algo_count(void) {
+    std::call_once(g_once, build_table);
+    return g_count;
+}
+
+extern "C" int fo_algo_info(int algo, int32_t info[12]) {
+    const fo_algo_entry *e = fo_algo_lookup(algo);
+    if (!e) return FO_ERR_ALGO;
+    if (!info) return FO_ERR_ARG;
+    for (int i = 0; i < 12; i++) info[i] = e->f[i];
+    return FO_OK;
+}
+
+extern "C" int fo_schedule_order(int algo, int M, int N, int32_t *order) {
+    if (!order) return FO_ERR_ARG;
+    fo_raster r;
+    int rc = fo_pick_raster(algo, M, N, &r);
+    if (rc) return rc;
+    const fo_algo_entry *e = fo_algo_lookup(algo);
+    const int bm = e->f[0], bn = e->f[1];
+    const int tn = N / bn;
+    const int sub_m = r.mtm / bm, sub_n = r.mtn / bn;
+    int k = 0;
+    for (int wg = 0; wg < r.grid_m * r.grid_n; wg++) {
+        int pm, pn;
+        fo_wg_to_tile(wg, r.grid_m, r.grid_n, r.panel, r.xcd_remap, &pm, &pn);
+        for (int s = 0; s < sub_m * sub_n; s++)
+            order[k++] = (pm * sub_m + s / sub_n) * tn + pn * sub_n + s % sub_n;
+    }
+    return FO_OK;
+}
+
+extern "C" int fo_version(void) { return 100; }
+
+extern "C" const char *fo_error_string(int code) {
+    switch (code) {
+        case FO_OK: return "ok";
+        case FO_ERR_ARG: return "null pointer or non-positive size";
+        case FO_ERR_SHAPE: return "shape not divisible by the tile (M % BM, N % BN, K % 64, dim % 8)";
+        case FO_ERR_ALGO: return "Algo index out of range";
+        case FO_ERR_DTYPE: return "dtype must be FO_F16 or FO_BF16";
+        case FO_ERR_SEGMENTS: return "cSeg does not partition the tiles (or too many groups for monitor mode)";
+        case FO_ERR_STATE: return "fo_overlap handle used before its init call";
+        default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
+    }
+}

@@ -1,0 +1,323 @@
+// Bandwidth-bound side kernels of the overlap path: counting/wait, the
+// consumer that stands in for the collective, and (reorder+)RMSNorm.
+#include <stdlib.h>
+
+#include "fo_common.h"
+
+namespace {
+
+// ------------------------------------------------------------------ wait
+// Replaces kernel_wait_flag (src/wait.cuh:5-9).  One lane polls with an
+// agent-scope acquire load and sleeps between polls; on equality a CAS resets
+// the counter to zero exactly as atomicCAS(addr, that, 0) does.
+__global__ void fo_wait_kernel(int expect, int32_t *counter, long max_polls, int32_t *status) {
+    long polls = 0;
+    for (;;) {
+        int v = __hip_atomic_load(counter, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+        if (v == expect) {
+            int e = expect;
+            if (__hip_atomic_compare_exchange_strong(counter, &e, 0, __ATOMIC_ACQ_REL,
+                                                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+                return;
+        }
+        if (max_polls > 0 && ++polls >= max_polls) {
+            if (status) __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return;
+        }
+        __builtin_amdgcn_s_sleep(8);
+    }
+}
+
+// ------------------------------------------------------------------ consumer
+template <typename Tag>
+__device__ __forceinline__ fo_u32x4 add8(fo_u32x4 a, fo_u32x4 b) {
+    typedef fo_elem<Tag> E;
+    uint32_t x[4] = {a.x, a.y, a.z, a.w}, y[4] = {b.x, b.y, b.z, b.w}, o[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float lo = E::to_f32((uint16_t)(x[i] & 0xffff)) + E::to_f32((uint16_t)(y[i] & 0xffff));
+        float hi = E::to_f32((uint16_t)(x[i] >> 16)) + E::to_f32((uint16_t)(y[i] >> 16));
+        o[i] = (uint32_t)E::from_f32(lo) | ((uint32_t)E::from_f32(hi) << 16);
+    }
+    return fo_u32x4{o[0], o[1], o[2], o[3]};
+}
+
+// acc[q*seg_stride + i] += src[q*chunk + i] for q < W, i < chunk (16-byte units).
+template <typename Tag>
+__global__ __launch_bounds__(256) void fo_consumer_kernel(const fo_u32x4 *src, fo_u32x4 *acc, long chunk16,
+                                                          int W, long seg_stride16) {
+    const long total = chunk16 * W;
+    const long step = (long)gridDim.x * blockDim.x;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += step) {
+        const long q = i / chunk16, o = i - q * chunk16;
+        fo_u32x4 *dst = acc + q * seg_stride16 + o;
+        *dst = add8<Tag>(*dst, src[i]);
+    }
+}
+
+// One launch for all groups: every workgroup, for each group in order, has one
+// lane wait for MM[g] == cseg[g] (acquire), then all its lanes reduce their
+// slice of the group's contiguous range.  No workgroup waits for another one;
+// the last workgroup to leave resets every group counter (the CAS-to-zero of
+// src/wait.cuh:5-9, deferred to the end of the launch, before which nothing can
+// signal again) and clears workspace word 0.  Word 1 is set if a bounded poll
+// gave up.
+template <typename Tag>
+__global__ __launch_bounds__(512) void fo_wait_reduce_kernel(const fo_u32x4 *C, fo_u32x4 *ACC, int32_t *MM,
+                                                             const int32_t *cseg, int G,
+                                                             long tile16, int W, long seg_stride16,
+                                                             int32_t *ws, long max_polls) {
+    const int nb = gridDim.x;
+    long base16 = 0;
+    for (int g = 0; g < G; g++) {
+        const int cnt = cseg[g];
+        if (threadIdx.x == 0) {
+            long polls = 0;
+            while (__hip_atomic_load(MM + g, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) != cnt) {
+                if (max_polls > 0 && ++polls >= max_polls) {  // debugging bound: flag and go on
+                    __hip_atomic_store(ws + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(4);
+            }
+        }
+        __syncthreads();
+        // The polling lane's acquire invalidated stale lines; repeat it for the
+        // other wavefronts' vector loads.
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        const long n16 = (long)cnt * tile16;
+        if (ACC) {
+            const long step = (long)nb * blockDim.x;
+            if (W <= 1) {
+                for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += step) {
+                    fo_u32x4 *dst = ACC + base16 + i;
+                    *dst = add8<Tag>(*dst, C[base16 + i]);
+                }
+            } else {
+                const long chunk16 = n16 / W;
+                for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += step) {
+                    const long q = i / chunk16, o = i - q * chunk16;
+                    fo_u32x4 *dst = ACC + q * seg_stride16 + base16 / W + o;
+                    *dst = add8<Tag>(*dst, C[base16 + i]);
+                }
+            }
+        }
+        base16 += n16;
+    }
+    __shared__ int last;
+    if (threadIdx.x == 0) {
+        int left = __hip_atomic_fetch_add(ws, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        last = (left == nb - 1);
+    }
+    __syncthreads();
+    if (last) {
+        for (int g = threadIdx.x; g < G; g += blockDim.x)
+            __hip_atomic_store(MM + g, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (threadIdx.x == 0) __hip_atomic_store(ws, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+// ------------------------------------------------------------------ RMSNorm
+// One wavefront per output row, four rows per workgroup; each lane keeps its
+// 16-byte chunks of the row in registers between the sum of squares and the
+// scaling, so the row is read once.  With RA != nullptr the chunks are gathered
+// from the tile-reordered buffer (index math of src/rmsnorm/rmsnorm.cuh:80-86).
+template <typename Tag, int MAXCH>
+__global__ __launch_bounds__(256) void fo_rmsnorm_kernel(const fo_u32x4 *X, fo_u32x4 *Y, const fo_u32x4 *Wt,
+                                                         int bs, int dim, int BM, int BN, int rldn,
+                                                         const int32_t *RA, float eps) {
+    typedef fo_elem<Tag> E;
+    const int lane = threadIdx.x & 63;
+    const int b = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (b >= bs) return;
+    const int nch = dim >> 3;  // 16-byte chunks per row
+    const int ldn = RA ? dim / BN : 0;
+    const int tile_row = RA ? b / BM : 0, in_row = RA ? b % BM : 0;
+    const long ldp16 = RA ? ((long)rldn * BN) >> 3 : 0;
+
+    fo_u32x4 x[MAXCH];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAXCH; i++) {
+        const int c = lane + i * 64;
+        if (c < nch) {
+            long src;
+            if (RA) {
+                const int j = c << 3;
+                const int r = RA[tile_row * ldn + j / BN];
+                const long nr = (long)(r / rldn) * BM + in_row;
+                const int nc = (r % rldn) * BN + j % BN;
+                src = nr * ldp16 + (nc >> 3);
+            } else {
+                src = (long)b * nch + c;
+            }
+            x[i] = X[src];
+            const uint32_t w[4] = {x[i].x, x[i].y, x[i].z, x[i].w};
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const float lo = E::to_f32((uint16_t)(w[k] & 0xffff));
+                const float hi = E::to_f32((uint16_t)(w[k] >> 16));
+                ss += lo * lo;
+                ss += hi * hi;
+            }
+        }
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) ss += __shfl_xor(ss, d, 64);
+    const float s = rsqrtf(ss / (float)dim + eps);
+
+#pragma unroll
+    for (int i = 0; i < MAXCH; i++) {
+        const int c = lane + i * 64;
+        if (c < nch) {
+            const fo_u32x4 wv = Wt[c];
+            const uint32_t xi[4] = {x[i].x, x[i].y, x[i].z, x[i].w};
+            const uint32_t wi[4] = {wv.x, wv.y, wv.z, wv.w};
+            uint32_t o[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                // y = round16(round16(x*s) * w): the second product is a 16-bit
+                // multiply in the reference (rmsnorm.cuh:110-112); the fp32
+                // product of two 16-bit values is exact, so one rounding matches.
+                const float lo = E::to_f32(E::from_f32(E::to_f32((uint16_t)(xi[k] & 0xffff)) * s));
+                const float hi = E::to_f32(E::from_f32(E::to_f32((uint16_t)(xi[k] >> 16)) * s));
+                const uint16_t ylo = E::from_f32(lo * E::to_f32((uint16_t)(wi[k] & 0xffff)));
+                const uint16_t yhi = E::from_f32(hi * E::to_f32((uint16_t)(wi[k] >> 16)));
+                o[k] = (uint32_t)ylo | ((uint32_t)yhi << 16);
+            }
+            Y[(long)b * nch + c] = fo_u32x4{o[0], o[1], o[2], o[3]};
+        }
+    }
+}
+
+template <typename Tag>
+int launch_rmsnorm(const void *X, void *Y, const void *Wt, int bs, int dim, int BM, int BN,
+                   int rldn, const int32_t *RA, float eps, hipStream_t stream) {
+    const int nch = dim / 8;
+    dim3 grid((bs + 3) / 4), block(256);
+    const fo_u32x4 *x = static_cast<const fo_u32x4 *>(X);
+    fo_u32x4 *y = static_cast<fo_u32x4 *>(Y);
+    const fo_u32x4 *w = static_cast<const fo_u32x4 *>(Wt);
+    if (nch <= 64 * 4)
+        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 4>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
+    else if (nch <= 64 * 8)
+        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 8>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
+    else if (nch <= 64 * 16)
+        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 16>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
+    else if (nch <= 64 * 32)
+        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 32>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
+    else
+        return FO_ERR_SHAPE;  // rows above 16384 elements (the reference's limit too)
+    FO_LAUNCH_CHECK();
+    return FO_OK;
+}
+
+// FO_WAIT_MAX_POLLS (environment, read once): bound for the otherwise unbounded
+// waits, so that a missing signal ends in a flagged exit instead of a hung GPU.
+long default_max_polls() {
+    static long v = [] {
+        const char *e = getenv("FO_WAIT_MAX_POLLS");
+        return e ? atol(e) : 0L;
+    }();
+    return v;
+}
+
+int consumer_grid(long n16) {
+    long blocks = (n16 + 256 * 4 - 1) / (256 * 4);  // about four 16-byte pieces per lane
+    if (blocks < 1) blocks = 1;
+    if (blocks > 2048) blocks = 2048;
+    return (int)blocks;
+}
+
+}  // namespace
+
+extern "C" int fo_wait(int expect, int32_t *counter, fo_stream_t stream) {
+    if (!counter) return FO_ERR_ARG;
+    hipLaunchKernelGGL(fo_wait_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream), expect,
+                       counter, default_max_polls(), (int32_t *)nullptr);
+    FO_LAUNCH_CHECK();
+    return FO_OK;
+}
+
+extern "C" int fo_wait_bounded(int expect, int32_t *counter, int64_t max_polls, int32_t *status,
+                               fo_stream_t stream) {
+    if (!counter || max_polls < 0) return FO_ERR_ARG;
+    hipLaunchKernelGGL(fo_wait_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream), expect,
+                       counter, (long)max_polls, status);
+    FO_LAUNCH_CHECK();
+    return FO_OK;
+}
+
+extern "C" int fo_consumer_reduce_rs(int dtype, const void *src, void *acc, int64_t nelem, int W,
+                                     int64_t seg_stride, fo_stream_t stream) {
+    if (!src || !acc || nelem < 0 || W <= 0) return FO_ERR_ARG;
+    if (nelem == 0) return FO_OK;
+    if (nelem % W || (nelem / W) % 8 || (W > 1 && seg_stride % 8)) return FO_ERR_SHAPE;
+    if (((uintptr_t)src | (uintptr_t)acc) & 15) return FO_ERR_SHAPE;
+    const long chunk16 = nelem / W / 8;
+    dim3 grid(consumer_grid(chunk16 * W)), block(256);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == FO_F16)
+        hipLaunchKernelGGL(fo_consumer_kernel<fo_f16_tag>, grid, block, 0, s, (const fo_u32x4 *)src,
+                           (fo_u32x4 *)acc, chunk16, W, (long)(seg_stride / 8));
+    else if (dtype == FO_BF16)
+        hipLaunchKernelGGL(fo_consumer_kernel<fo_bf16_tag>, grid, block, 0, s, (const fo_u32x4 *)src,
+                           (fo_u32x4 *)acc, chunk16, W, (long)(seg_stride / 8));
+    else
+        return FO_ERR_DTYPE;
+    FO_LAUNCH_CHECK();
+    return FO_OK;
+}
+
+extern "C" int fo_consumer_reduce(int dtype, const void *src, void *acc, int64_t nelem,
+                                  fo_stream_t stream) {
+    return fo_consumer_reduce_rs(dtype, src, acc, nelem, 1, 0, stream);
+}
+
+extern "C" int fo_wait_reduce_groups(int dtype, const void *C, void *ACC, int32_t *MM,
+                                     const int32_t *cseg_dev, int G, int64_t tile_elems, int W,
+                                     int64_t seg_stride, int32_t *workspace, int nblocks,
+                                     fo_stream_t stream) {
+    if (!MM || !cseg_dev || !workspace || G <= 0 || tile_elems <= 0 || W <= 0) return FO_ERR_ARG;
+    if (ACC && !C) return FO_ERR_ARG;
+    if (tile_elems % (8 * W) || (W > 1 && seg_stride % 8)) return FO_ERR_SHAPE;
+    if (nblocks <= 0) nblocks = 32;
+    if (nblocks > 256) nblocks = 256;
+    dim3 grid(nblocks), block(512);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == FO_F16)
+        hipLaunchKernelGGL(fo_wait_reduce_kernel<fo_f16_tag>, grid, block, 0, s, (const fo_u32x4 *)C,
+                           (fo_u32x4 *)ACC, MM, cseg_dev, G, (long)(tile_elems / 8), W,
+                           (long)(seg_stride / 8), workspace, default_max_polls());
+    else if (dtype == FO_BF16)
+        hipLaunchKernelGGL(fo_wait_reduce_kernel<fo_bf16_tag>, grid, block, 0, s, (const fo_u32x4 *)C,
+                           (fo_u32x4 *)ACC, MM, cseg_dev, G, (long)(tile_elems / 8), W,
+                           (long)(seg_stride / 8), workspace, default_max_polls());
+    else
+        return FO_ERR_DTYPE;
+    FO_LAUNCH_CHECK();
+    return FO_OK;
+}
+
+extern "C" int fo_reorder_rmsnorm(int dtype, const void *X, void *Y, const void *Wt, int bs, int dim,
+                                  int BM, int BN, int rldn, const int32_t *RA, float eps,
+                                  fo_stream_t stream) {
+    if (!X || !Y || !Wt || !RA || bs <= 0 || dim <= 0 || BM <= 0 || BN <= 0 || rldn <= 0)
+        return FO_ERR_ARG;
+    if (dim % 8 || BN % 8 || dim % BN || bs % BM) return FO_ERR_SHAPE;
+    if (((long)(bs / BM) * (dim / BN)) % rldn) return FO_ERR_SHAPE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == FO_F16) return launch_rmsnorm<fo_f16_tag>(X, Y, Wt, bs, dim, BM, BN, rldn, RA, eps, s);
+    if (dtype == FO_BF16) return launch_rmsnorm<fo_bf16_tag>(X, Y, Wt, bs, dim, BM, BN, rldn, RA, eps, s);
+    return FO_ERR_DTYPE;
+}
+
+extern "C" int fo_rmsnorm(int dtype, const void *X, void *Y, const void *Wt, int bs, int dim,
+                          float eps, fo_stream_t stream) {
+    if (!X || !Y || !Wt || bs <= 0 || dim <= 0) return FO_ERR_ARG;
+    if (dim % 8) return FO_ERR_SHAPE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == FO_F16) return launch_rmsnorm<fo_f16_tag>(X, Y, Wt, bs, dim, 1, 8, 1, nullptr, eps, s);
+    if (dtype == FO_BF16) return launch_rmsnorm<fo_bf16_tag>(X, Y, Wt, bs, dim, 1, 8, 1, nullptr, eps, s);
+    return FO_ERR_DTYPE;
+}

@@ -1,0 +1,96 @@
+// Shared declarations of the gfx950 kernel library (internal; the public C ABI
+// is include/flashoverlap.h).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "flashoverlap.h"
+
+#define FO_HIP_CHECK(expr)                        \
+    do {                                          \
+        hipError_t e__ = (expr);                  \
+        if (e__ != hipSuccess) return (int)e__;   \
+    } while (0)
+
+// The launch itself reports configuration errors through hipGetLastError.
+#define FO_LAUNCH_CHECK()                         \
+    do {                                          \
+        hipError_t e__ = hipGetLastError();       \
+        if (e__ != hipSuccess) return (int)e__;   \
+    } while (0)
+
+typedef _Float16 fo_half8 __attribute__((ext_vector_type(8)));
+typedef __bf16 fo_bf8 __attribute__((ext_vector_type(8)));
+typedef float fo_float16v __attribute__((ext_vector_type(16)));
+// Native 16- and 8-byte vectors (HIP's uint4 is a struct that register promotion handles badly).
+typedef unsigned int fo_u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int fo_u32x2 __attribute__((ext_vector_type(2)));
+
+struct fo_f16_tag {};
+struct fo_bf16_tag {};
+
+// 16-bit <-> fp32 element conversions (round to nearest even, hardware cvt).
+template <typename Tag> struct fo_elem;
+template <> struct fo_elem<fo_f16_tag> {
+    typedef _Float16 type;
+    typedef fo_half8 vec8;
+    static __device__ __forceinline__ float to_f32(uint16_t b) {
+        return (float)__builtin_bit_cast(_Float16, b);
+    }
+    static __device__ __forceinline__ uint16_t from_f32(float f) {
+        return __builtin_bit_cast(uint16_t, (_Float16)f);
+    }
+    static __device__ __forceinline__ fo_float16v mfma(fo_u32x4 a, fo_u32x4 b, fo_float16v c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(fo_half8, a),
+                                                      __builtin_bit_cast(fo_half8, b), c, 0, 0, 0);
+    }
+};
+template <> struct fo_elem<fo_bf16_tag> {
+    typedef __bf16 type;
+    typedef fo_bf8 vec8;
+    static __device__ __forceinline__ float to_f32(uint16_t b) {
+        return __builtin_bit_cast(float, (uint32_t)b << 16);
+    }
+    static __device__ __forceinline__ uint16_t from_f32(float f) {
+        return __builtin_bit_cast(uint16_t, (__bf16)f);
+    }
+    static __device__ __forceinline__ fo_float16v mfma(fo_u32x4 a, fo_u32x4 b, fo_float16v c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(fo_bf8, a),
+                                                       __builtin_bit_cast(fo_bf8, b), c, 0, 0, 0);
+    }
+};
+
+// Algo table (fo_algo.cpp).
+struct fo_algo_entry {
+    int32_t f[12];  // TbM,TbN,TbK,WarpM,WarpN,WarpK,InstM,InstN,InstK,Stages,Swizzle,SplitK
+};
+const fo_algo_entry *fo_algo_lookup(int algo);
+
+// Macro-tile choice and raster shared by the launcher and fo_schedule_order.
+struct fo_raster {
+    int mtm, mtn;        // macro tile (workgroup tile) in elements
+    int grid_m, grid_n;  // macro tiles along M and N
+    int panel;           // raster panel height in macro tiles
+    int xcd_remap;       // 1: workgroup id is de-interleaved over the 8 XCDs
+};
+int fo_pick_raster(int algo, int M, int N, fo_raster *r);
+
+// Workgroup id -> macro tile coordinates; identical code on host and device.
+__host__ __device__ inline void fo_wg_to_tile(int wg, int grid_m, int grid_n, int panel,
+                                              int xcd_remap, int *pm, int *pn) {
+    int nt = grid_m * grid_n;
+    int v = wg;
+    if (xcd_remap) {
+        // Workgroups are dealt round-robin to the 8 XCDs; give each XCD one
+        // contiguous range of the raster so its private L2 sees neighbouring tiles.
+        v = (wg & 7) * (nt >> 3) + (wg >> 3);
+    }
+    int per_panel = panel * grid_n;
+    int p = v / per_panel;
+    int first_m = p * panel;
+    int rows = grid_m - first_m < panel ? grid_m - first_m : panel;
+    int in = v - p * per_panel;
+    *pm = first_m + in % rows;
+    *pn = in / rows;
+}

@@ -1,0 +1,240 @@
+// Host orchestration of the overlap path: the counterpart of class OverlapImpl
+// (src/overlap_impl.h:12-43, src/overlap_impl.cu) behind a C handle.  Two HIP
+// streams and one event; every call only enqueues work and returns.
+#include <new>
+
+#include "fo_common.h"
+
+struct fo_overlap {
+    hipStream_t gemm_stream = nullptr;
+    hipStream_t comm_stream = nullptr;
+    hipEvent_t joined = nullptr;
+    int32_t *workspace = nullptr;  // one zeroed word for the fused wait+reduce kernel
+    bool gemm_ready = false;
+    bool overlap_ready = false;
+    int rank = 0, world = 1;
+    void *acc = nullptr;
+    int64_t acc_nelem = 0;
+    int fused = 0;
+};
+
+namespace {
+
+int check_segments(const int32_t *cseg_host, int G, long tiles) {
+    if (!cseg_host || G <= 0) return FO_ERR_SEGMENTS;
+    long sum = 0;
+    for (int i = 0; i < G; i++) {
+        if (cseg_host[i] <= 0) return FO_ERR_SEGMENTS;
+        sum += cseg_host[i];
+    }
+    return sum == tiles ? FO_OK : FO_ERR_SEGMENTS;
+}
+
+// consumer stream -> GEMM stream, as the event pair at src/overlap_impl.cu:260-263.
+int join(fo_overlap *h) {
+    FO_HIP_CHECK(hipEventRecord(h->joined, h->comm_stream));
+    FO_HIP_CHECK(hipStreamWaitEvent(h->gemm_stream, h->joined, 0));
+    return FO_OK;
+}
+
+}  // namespace
+
+extern "C" int fo_overlap_create(fo_overlap_t **out) {
+    if (!out) return FO_ERR_ARG;
+    *out = new (std::nothrow) fo_overlap();
+    return *out ? FO_OK : FO_ERR_ARG;
+}
+
+extern "C" int fo_overlap_destroy(fo_overlap_t *h) {
+    if (!h) return FO_ERR_ARG;
+    if (h->comm_stream) {
+        hipStreamSynchronize(h->comm_stream);
+        hipStreamDestroy(h->comm_stream);
+    }
+    if (h->joined) hipEventDestroy(h->joined);
+    if (h->workspace) hipFree(h->workspace);
+    delete h;
+    return FO_OK;
+}
+
+extern "C" int fo_overlap_set_gemm_stream(fo_overlap_t *h, fo_stream_t gemm_stream) {
+    if (!h) return FO_ERR_ARG;
+    h->gemm_stream = static_cast<hipStream_t>(gemm_stream);
+    h->gemm_ready = true;
+    return FO_OK;
+}
+
+extern "C" int fo_overlap_init(fo_overlap_t *h) {
+    if (!h) return FO_ERR_ARG;
+    if (h->overlap_ready) return FO_OK;
+    // Default priority on purpose (the reference asks for priority -5,
+    // src/overlap_impl.cu:140): mixed-priority streams are avoided on this platform.
+    FO_HIP_CHECK(hipStreamCreateWithFlags(&h->comm_stream, hipStreamNonBlocking));
+    FO_HIP_CHECK(hipEventCreateWithFlags(&h->joined, hipEventDisableTiming));
+    FO_HIP_CHECK(hipMalloc(&h->workspace, 64));
+    FO_HIP_CHECK(hipMemset(h->workspace, 0, 64));
+    h->overlap_ready = true;
+    return FO_OK;
+}
+
+extern "C" int fo_overlap_set_world(fo_overlap_t *h, int rank, int world) {
+    if (!h || world <= 0 || rank < 0 || rank >= world) return FO_ERR_ARG;
+    h->rank = rank;
+    h->world = world;
+    return FO_OK;
+}
+
+extern "C" int fo_overlap_set_accumulator(fo_overlap_t *h, void *acc, int64_t nelem) {
+    if (!h || nelem < 0) return FO_ERR_ARG;
+    h->acc = acc;
+    h->acc_nelem = acc ? nelem : 0;
+    return FO_OK;
+}
+
+extern "C" int fo_overlap_set_fused_consumer(fo_overlap_t *h, int fused) {
+    if (!h) return FO_ERR_ARG;
+    h->fused = fused ? 1 : 0;
+    return FO_OK;
+}
+
+extern "C" fo_stream_t fo_overlap_comm_stream(fo_overlap_t *h) {
+    return h ? static_cast<fo_stream_t>(h->comm_stream) : nullptr;
+}
+
+extern "C" int fo_overlap_gemm(fo_overlap_t *h, int dtype, int M, int N, int K, const void *A,
+                               const void *B, void *C, int algo) {
+    if (!h) return FO_ERR_ARG;
+    if (!h->gemm_ready) return FO_ERR_STATE;
+    return fo_gemm(dtype, M, N, K, A, B, C, algo, h->gemm_stream);
+}
+
+extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int N, int K,
+                                         const void *A, const void *B, void *C, int32_t *MM,
+                                         const int32_t *RA, int TM, int TN, int rLDN,
+                                         const int32_t *cseg_host, const int32_t *cseg_dev, int G,
+                                         int algo, int monitor) {
+    if (!h) return FO_ERR_ARG;
+    if (!h->gemm_ready || !h->overlap_ready) return FO_ERR_STATE;
+    int32_t info[12];
+    int rc = fo_algo_info(algo, info);
+    if (rc) return rc;
+    if (M <= 0 || N <= 0 || M % info[0] || N % info[1]) return FO_ERR_SHAPE;
+    if (TM != M / info[0] || TN != N / info[1]) return FO_ERR_SHAPE;  // RA.shape must match the Algo's tile
+    rc = check_segments(cseg_host, G, (long)TM * TN);
+    if (rc) return rc;
+    const int64_t tile_elems = (int64_t)info[0] * info[1];
+    if (h->acc && h->acc_nelem < (int64_t)M * N) return FO_ERR_ARG;
+
+    rc = fo_gemm_signal(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, MM, RA, monitor, algo,
+                        h->gemm_stream);
+    if (rc) return rc;  // nothing has been enqueued on the consumer stream yet
+
+    if (h->fused) {
+        rc = fo_wait_reduce_groups(dtype, C, h->acc, MM, cseg_dev, G, tile_elems, 1, 0, h->workspace,
+                                   0, h->comm_stream);
+        if (rc) return rc;
+    } else {
+        int64_t off = 0;
+        uint16_t *c = static_cast<uint16_t *>(C);
+        uint16_t *acc = static_cast<uint16_t *>(h->acc);
+        for (int i = 0; i < G; i++) {
+            const int64_t n = cseg_host[i] * tile_elems;
+            rc = fo_wait(cseg_host[i], MM + i, h->comm_stream);  // resets the counter
+            if (rc) return rc;
+            if (acc) {
+                rc = fo_consumer_reduce(dtype, c + off, acc + off, n, h->comm_stream);
+                if (rc) return rc;
+            }
+            off += n;
+        }
+    }
+    return join(h);
+}
+
+extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, int N, int K,
+                                             const void *A, const void *B, void *C, void *D,
+                                             int32_t *MM, const int32_t *RA, const int32_t *RE,
+                                             int TM, int TN, int rLDN, const int32_t *cseg_host,
+                                             const int32_t *cseg_dev, int G, int algo, int monitor) {
+    if (!h) return FO_ERR_ARG;
+    if (!h->gemm_ready || !h->overlap_ready) return FO_ERR_STATE;
+    int32_t info[12];
+    int rc = fo_algo_info(algo, info);
+    if (rc) return rc;
+    if (M <= 0 || N <= 0 || M % info[0] || N % info[1]) return FO_ERR_SHAPE;
+    if (TM != M / info[0] || TN != N / info[1]) return FO_ERR_SHAPE;
+    rc = check_segments(cseg_host, G, (long)TM * TN);
+    if (rc) return rc;
+    const int W = h->world;
+    const int64_t tile_elems = (int64_t)info[0] * info[1];
+    if (tile_elems % (8 * W) || ((int64_t)M * N) % W) return FO_ERR_SHAPE;
+    const int64_t seg_stride = (int64_t)M * N / W;
+    if (h->acc && h->acc_nelem < (int64_t)M * N) return FO_ERR_ARG;
+
+    rc = fo_gemm_scatter(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, MM, RA, RE, monitor, algo,
+                         h->gemm_stream);
+    if (rc) return rc;
+
+    uint16_t *c = static_cast<uint16_t *>(C);
+    uint16_t *d = static_cast<uint16_t *>(D);
+    uint16_t *acc = static_cast<uint16_t *>(h->acc);
+    if (h->fused) {
+        rc = fo_wait_reduce_groups(dtype, C, h->acc, MM, cseg_dev, G, tile_elems, W, seg_stride,
+                                   h->workspace, 0, h->comm_stream);
+        if (rc) return rc;
+    }
+    int64_t off = 0;
+    for (int i = 0; i < G; i++) {
+        const int64_t n = cseg_host[i] * tile_elems;
+        if (!h->fused) {
+            rc = fo_wait(cseg_host[i], MM + i, h->comm_stream);
+            if (rc) return rc;
+            if (acc) {
+                rc = fo_consumer_reduce_rs(dtype, c + off, acc + off / W, n, W, seg_stride,
+                                           h->comm_stream);
+                if (rc) return rc;
+            }
+        }
+        // ncclReduceScatter(C+acc -> D+acc/W, n/W) with one rank present: this
+        // rank's chunk of the group is the sum (src/overlap_impl.cu:312-313).
+        if (d)
+            FO_HIP_CHECK(hipMemcpyAsync(d + off / W, c + off + (int64_t)h->rank * (n / W),
+                                        (size_t)(n / W) * 2, hipMemcpyDeviceToDevice,
+                                        h->comm_stream));
+        off += n;
+    }
+    return join(h);
+}
+
+extern "C" int fo_overlap_gemm_allreduce_serial(fo_overlap_t *h, int dtype, int M, int N, int K,
+                                                const void *A, const void *B, void *C, int algo) {
+    if (!h) return FO_ERR_ARG;
+    if (!h->gemm_ready) return FO_ERR_STATE;
+    if (h->acc && h->acc_nelem < (int64_t)M * N) return FO_ERR_ARG;
+    int rc = fo_gemm(dtype, M, N, K, A, B, C, algo, h->gemm_stream);
+    if (rc) return rc;
+    if (h->acc) return fo_consumer_reduce(dtype, C, h->acc, (int64_t)M * N, h->gemm_stream);
+    return FO_OK;
+}
+
+extern "C" int fo_overlap_seg_allreduce(fo_overlap_t *h, int dtype, void *C, int64_t MN,
+                                        const int32_t *cseg_host, int G, int seg_num) {
+    if (!h || !C || !cseg_host || G <= 0 || seg_num <= 0 || MN <= 0) return FO_ERR_ARG;
+    if (!h->gemm_ready) return FO_ERR_STATE;
+    if (MN % seg_num || G < seg_num) return FO_ERR_SHAPE;
+    if (h->acc && h->acc_nelem < MN) return FO_ERR_ARG;
+    const int64_t unit = MN / seg_num;
+    int64_t off = 0;
+    uint16_t *c = static_cast<uint16_t *>(C);
+    uint16_t *acc = static_cast<uint16_t *>(h->acc);
+    for (int s = 0; s < seg_num; s++) {  // the reference iterates SegNum times over cSEG_CPU
+        const int64_t n = unit * cseg_host[s];
+        if (off + n > MN) return FO_ERR_SEGMENTS;
+        if (acc) {
+            int rc = fo_consumer_reduce(dtype, c + off, acc + off, n, h->gemm_stream);
+            if (rc) return rc;
+        }
+        off += n;
+    }
+    return FO_OK;
+}

@@ -1,0 +1,220 @@
+"""Wave-group tuning for one GPU: GEMM tile candidates, completion-order hint,
+consumer bandwidth curve, exhaustive and predictive search.
+
+Counterpart of tune/gen_config.py:25-86 (GEMM candidates), tune/bandwidth.py:77-111
+(size -> bandwidth curve, here of the consumer kernel instead of NCCL),
+tune/search.py:83-157 (hint from monitor mode), :180-235 (latency model),
+:376-385 (compositions), :387-502 (searches).  The latency model is written for
+the general "communication stage with a measured bandwidth curve"; the caller
+says how many bytes the stage moves per element.
+"""
+import numpy as np
+import torch
+
+from . import _capi, ops
+from .layout import cseg_from_waves, div_up, reorder_indices, counter_size
+
+CONSUMER_BYTES_PER_ELEM = 6.0  # read group + read accumulator + write accumulator, 16-bit each
+
+
+# ------------------------------------------------------------------ model
+def interpolate_latency(curve, x, bytes_per_elem=CONSUMER_BYTES_PER_ELEM):
+    """ms for a stage over x elements; curve[:,0] = elements, curve[:,1] = GiB/ms,
+    linear interpolation clamped at both ends (tune/search.py:180-205; there the
+    byte factor is 2*2*(W-1) for all_reduce and 2*(W-1) for reduce_scatter)."""
+    curve = np.asarray(curve, dtype=np.float64)
+    bw = float(np.interp(float(x), curve[:, 0], curve[:, 1]))
+    return float(x) * bytes_per_elem / bw / (1024 ** 3)
+
+
+def predict_latency(M, N, gemm_dur, curve, gp, tile_num, wave, full_wave=None,
+                    bytes_per_elem=CONSUMER_BYTES_PER_ELEM):
+    """Pipeline model of tune/search.py:207-235.  `wave` = tiles per wave while the
+    second stream is busy (reference: sm_count-2), `full_wave` = tiles per wave
+    of the GEMM alone (reference: sm_count)."""
+    full_wave = full_wave or wave
+    per_tile = M * N // tile_num
+    if len(gp) == 1:
+        return interpolate_latency(curve, per_tile * gp[0], bytes_per_elem) + gemm_dur
+    old_waves = div_up(tile_num, full_wave)
+    new_waves = div_up(tile_num, wave)
+    gemm = gemm_dur / old_waves * new_waves
+    acc_comm = acc_comp = 0.0
+    for i, g in enumerate(gp):
+        comm = 0.0 if i == 0 else interpolate_latency(curve, per_tile * gp[i - 1], bytes_per_elem)
+        acc_comm = max(acc_comp, acc_comm) + comm
+        acc_comp += gemm / new_waves * div_up(g, wave)
+    return max(acc_comp, acc_comm) + interpolate_latency(curve, per_tile * gp[-1], bytes_per_elem)
+
+
+def integer_partitions(n):
+    """All compositions (ordered partitions) of n, first part ascending
+    (tune/search.py:376-385; 2^(n-1) of them)."""
+    out = []
+
+    def rec(rem, path):
+        if rem == 0:
+            out.append(path)
+            return
+        for i in range(1, rem + 1):
+            rec(rem - i, path + [i])
+
+    rec(n, [])
+    return out
+
+
+def groups_to_cseg(gp, unit, tile_num):
+    """Scale a composition (in units of `unit` tiles) to tile counts; the last
+    group takes what is left (tune/search.py:423-429, :484-490)."""
+    cseg, acc = [], 0
+    for j, g in enumerate(gp):
+        if j < len(gp) - 1:
+            cseg.append(g * unit)
+            acc += g * unit
+        else:
+            cseg.append(min(g * unit, tile_num - acc))
+    return cseg
+
+
+def predictive_search(M, N, gemm_dur, curve, tile_num, wave, full_wave=None,
+                      bytes_per_elem=CONSUMER_BYTES_PER_ELEM):
+    """Best cSeg under the model (tune/search.py:442-502 without the measuring
+    steps): groups are multiples of min_group = ceil(wave_num/10) waves, long
+    splits with a big first group are skipped ("cold start")."""
+    wave_num = div_up(tile_num, wave)
+    min_group = div_up(wave_num, 10)
+    best, best_dur = None, float("inf")
+    for gp in integer_partitions(div_up(wave_num, min_group)):
+        if len(gp) > 5 and gp[0] > 2:
+            continue
+        cseg = groups_to_cseg(gp, wave * min_group, tile_num)
+        if min(cseg) <= 0:
+            continue
+        dur = predict_latency(M, N, gemm_dur, curve, cseg, tile_num, wave, full_wave, bytes_per_elem)
+        if dur < best_dur:
+            best, best_dur = cseg, dur
+    return best, best_dur
+
+
+# ------------------------------------------------------------------ measurement (GPU)
+def _time_ms(fn, warmup, reps):
+    for _ in range(warmup):
+        fn()
+    start = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
+    end = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
+    for i in range(reps):
+        start[i].record()
+        fn()
+        end[i].record()
+    torch.cuda.synchronize()
+    return float(np.mean([s.elapsed_time(e) for s, e in zip(start, end)]))
+
+
+def profile_gemm_configs(M, N, K, dtype=torch.float16, top=10, warmup=10, reps=100):
+    """Time every Algo whose tile divides the shape and return the stage-1 lists
+    (BM, BN, dur ms, Algo) of the `top` fastest (tune/gen_config.py:25-67)."""
+    A = torch.randn(M, K, device="cuda").to(dtype)
+    B = torch.randn(N, K, device="cuda").to(dtype)
+    C = torch.empty(M, N, device="cuda", dtype=dtype)
+    rows = []
+    for algo, row in enumerate(_capi.algo_table()):
+        if M % row[0] or N % row[1]:
+            continue
+        rows.append((_time_ms(lambda: ops.gemm(A, B, C, algo), warmup, reps), row[0], row[1], algo))
+    rows.sort()
+    rows = rows[:top]
+    return [r[1] for r in rows], [r[2] for r in rows], [r[0] for r in rows], [r[3] for r in rows]
+
+
+def consumer_bandwidth_curve(dtype=torch.float16, points=36, warmup=5, reps=20):
+    """[points, 2] tensor (elements, GiB/ms) of the consumer over 2^(20+0.25 i)
+    elements -- the one-GPU analogue of tune/bandwidth.py:77-111."""
+    sizes = [int(2 ** (20 + 0.25 * i)) // 8 * 8 for i in range(points)]
+    buf = torch.zeros(max(sizes), device="cuda", dtype=dtype)
+    acc = torch.zeros(max(sizes), device="cuda", dtype=dtype)
+    out = torch.empty(points, 2, dtype=torch.float64)
+    for i, n in enumerate(sizes):
+        ms = _time_ms(lambda: ops.consumer_reduce(buf[:n], acc[:n]), warmup, reps)
+        out[i, 0] = n
+        out[i, 1] = n * CONSUMER_BYTES_PER_ELEM / (1024 ** 3) / ms
+    return out
+
+
+def measured_hint(M, N, K, algo, wave, dtype=torch.float16, warmup=20, samples=10):
+    """Completion-order hint from monitor mode with the reference's consistency
+    rule: a tile belongs to wave w only if its stamp fell in
+    [w*wave, (w+1)*wave) in every sample, and every wave but the last must be
+    full (tune/search.py:96-157).  Returns (consistent, hint)."""
+    BM, BN = _capi.algo_tile(algo)
+    TM, TN = M // BM, N // BN
+    T = TM * TN
+    cseg = cseg_from_waves(T, wave)
+    if len(cseg) > TN - 1:
+        raise ValueError("monitor mode needs fewer groups than tile columns")
+    cseg_cpu = torch.tensor(cseg, dtype=torch.int32)
+    cseg_gpu = cseg_cpu.cuda()
+    A = torch.randn(M, K, device="cuda").to(dtype)
+    B = torch.randn(N, K, device="cuda").to(dtype)
+    C = torch.empty(M, N, device="cuda", dtype=dtype)
+    MM = torch.zeros((TM + 1, TN), dtype=torch.int32, device="cuda")
+    RA = torch.arange(T, dtype=torch.int32, device="cuda").reshape(TM, TN)
+    ov = ops.Overlap()
+    for _ in range(warmup):
+        ov.gemm_allreduce_overlap(A, B, C, MM, RA, 1, cseg_cpu, cseg_gpu, algo, True)
+    stamps = torch.empty((samples, T), dtype=torch.int32, device="cuda")
+    for i in range(samples):
+        torch.cuda.synchronize()
+        MM[0] = 0
+        ov.gemm_allreduce_overlap(A, B, C, MM, RA, 1, cseg_cpu, cseg_gpu, algo, True)
+        torch.cuda.synchronize()
+        stamps[i] = MM[1:].reshape(-1)
+    ov.close()
+    hint, ok = [], True
+    for w in range(len(cseg)):
+        inside = ((stamps >= w * wave) & (stamps < (w + 1) * wave)).sum(dim=0) == samples
+        idx = torch.where(inside)[0]
+        if w < len(cseg) - 1 and idx.numel() < wave:
+            ok = False
+            break
+        hint += idx.tolist()
+    return ok, hint
+
+
+def time_overlap(M, N, K, algo, cseg, hint, dtype=torch.float16, warmup=20, reps=200, fused=False,
+                 with_consumer=True):
+    """Mean ms of the overlapped call for one cSeg (tune/search.py:255-347)."""
+    BM, BN = _capi.algo_tile(algo)
+    TM, TN = M // BM, N // BN
+    A = torch.randn(M, K, device="cuda").to(dtype)
+    B = torch.randn(N, K, device="cuda").to(dtype)
+    C = torch.empty(M, N, device="cuda", dtype=dtype)
+    MM = torch.zeros(counter_size(len(cseg), TM, TN), dtype=torch.int32, device="cuda")
+    RA = reorder_indices(TM * TN, hint).reshape(TM, TN)
+    cseg_cpu = torch.tensor(cseg, dtype=torch.int32)
+    cseg_gpu = cseg_cpu.cuda()
+    ov = ops.Overlap()
+    ov.set_fused_consumer(fused)
+    if with_consumer:
+        ov.set_accumulator(torch.zeros(M * N, device="cuda", dtype=dtype))
+    if len(cseg) == 1:
+        ms = _time_ms(lambda: ov.gemm_allreduce(A, B, C, algo), warmup, reps)
+    else:
+        ms = _time_ms(lambda: ov.gemm_allreduce_overlap(A, B, C, MM, RA, 1, cseg_cpu, cseg_gpu, algo),
+                      warmup, reps)
+    torch.cuda.synchronize()
+    ov.close()
+    return ms
+
+
+def exhaustive_search(M, N, K, algo, wave, hint, dtype=torch.float16, reps=50):
+    """Measure every composition of the wave count (tune/search.py:387-439)."""
+    BM, BN = _capi.algo_tile(algo)
+    tile_num = (M // BM) * (N // BN)
+    best, best_ms, table = None, float("inf"), []
+    for gp in integer_partitions(div_up(tile_num, wave)):
+        cseg = groups_to_cseg(gp, wave, tile_num)
+        ms = time_overlap(M, N, K, algo, cseg, hint, dtype, warmup=5, reps=reps)
+        table.append((cseg, ms))
+        if ms < best_ms:
+            best, best_ms = cseg, ms
+    return best, best_ms, table

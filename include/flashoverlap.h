@@ -1,0 +1,199 @@
+/*
+ * flashoverlap.h -- C ABI of the MI355X (gfx950) FlashOverlap hot path.
+ *
+ * libfo_kernels.so exports exactly these symbols.  Plain pointers and sizes
+ * only; every pointer named "device" must be HIP device memory on the current
+ * device, every fo_stream_t is a hipStream_t (NULL = the null stream).  All
+ * work is enqueued asynchronously; nothing here allocates device memory
+ * except fo_overlap_create/fo_overlap_init (one stream) and the optional
+ * workspace noted below.
+ *
+ * Return value: 0 = ok, <0 = argument error (FO_ERR_*), >0 = hipError_t.
+ *
+ * Each declaration cites the interface of infinigence/FlashOverlap that it
+ * replaces (path:line in that tree).
+ */
+#ifndef FLASHOVERLAP_H
+#define FLASHOVERLAP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *fo_stream_t; /* hipStream_t */
+
+enum { FO_F16 = 0, FO_BF16 = 1 };
+
+enum {
+    FO_OK = 0,
+    FO_ERR_ARG = -1,      /* null pointer / non-positive size */
+    FO_ERR_SHAPE = -2,    /* M % BM, N % BN, K % 64, dim % 8 ... violated */
+    FO_ERR_ALGO = -3,     /* Algo outside [0, fo_algo_count()) */
+    FO_ERR_DTYPE = -4,    /* dtype not FO_F16 / FO_BF16 */
+    FO_ERR_SEGMENTS = -5, /* sum(cSeg) != tile count, G <= 0, monitor with G > TN-1 */
+    FO_ERR_STATE = -6     /* fo_overlap_* called before the matching init */
+};
+
+const char *fo_error_string(int code);
+int fo_version(void);
+
+/* ---- Algo index space -------------------------------------------------
+ * Same 102-entry index space as the generated function-pointer tables
+ * src/tiling/gemm_tiling.cuh:3-106 / signal_tiling.cuh / scatter_tiling.cuh
+ * (generator tool/generate_instances.py:5-37).  info[12] =
+ * {TbM,TbN,TbK,WarpM,WarpN,WarpK,InstM,InstN,InstK,Stages,Swizzle,SplitK}.
+ * On gfx950 (TbM,TbN) are the reorder/signal tile BM x BN and Swizzle is the
+ * raster panel height; the other fields are advisory. */
+int fo_algo_count(void);
+int fo_algo_info(int algo, int32_t info[12]);
+
+/* Tile issue order of the GEMM kernels: order[s] = id (tm*TN + tn) of the
+ * s-th BM x BN tile in workgroup dispatch order.  It is the analytic
+ * counterpart of the hint that tune/search.py:83-157 measures in monitor
+ * mode; order must hold (M/BM)*(N/BN) ints (host memory). */
+int fo_schedule_order(int algo, int M, int N, int32_t *order);
+
+/* ---- GEMM -------------------------------------------------------------
+ * C[M,N] = A[M,K] . B[N,K]^T, 16-bit in/out, fp32 accumulate.
+ * Replaces gemm_func_table[Algo](M,N,K,A,B,C,stream), src/gemm/gemm.cu:23-110,
+ * typedef src/tiling/gemm_dispatcher.h:7-26. Requires M % TbM == 0,
+ * N % TbN == 0, K % 64 == 0 (the reference has no boundary handling either,
+ * README.md:73). */
+int fo_gemm(int dtype, int M, int N, int K, const void *A, const void *B, void *C, int algo,
+            fo_stream_t stream);
+
+/* GEMM + reordered tile store + per-group signal.
+ * Replaces signal_func_table[Algo](M,N,K,rLDN,cSeg,A,B,C,MM,RA,if_monitor,stream),
+ * src/overlap/gemm_signal.cu:15-97 (epilogue src/overlap/gemm_with_signal.h:236-256,
+ * :291-361).  RA[TM*TN], cseg_dev[G], MM[>= G; monitor: (TM+1)*TN] are device
+ * int32.  Tile t is stored at slot r = RA[t] of C viewed as
+ * [(M*N)/(rLDN*BN), rLDN*BN]; after the tile's stores are released at agent
+ * scope, MM[group(r)] += 1; monitor: o = MM[TN-1]++, MM[TN+r] = o.
+ * G is an extra argument (the reference reads cSeg until the prefix sum passes
+ * r); it lets the library validate on the host when cseg_host != NULL. */
+int fo_gemm_signal(int dtype, int M, int N, int K, int rLDN, const int32_t *cseg_dev, int G,
+                   const void *A, const void *B, void *C, int32_t *MM, const int32_t *RA,
+                   int monitor, int algo, fo_stream_t stream);
+
+/* As fo_gemm_signal, and row rho of the reshaped C goes to row RE[rho].
+ * Replaces scatter_func_table[Algo](...,RE,...), src/overlap/gemm_scatter.cu:15-98
+ * (src/overlap/gemm_with_scatter.h:229, :448-473). RE[(M*N)/(rLDN*BN)] device int32. */
+int fo_gemm_scatter(int dtype, int M, int N, int K, int rLDN, const int32_t *cseg_dev, int G,
+                    const void *A, const void *B, void *C, int32_t *MM, const int32_t *RA,
+                    const int32_t *RE, int monitor, int algo, fo_stream_t stream);
+
+/* ---- counting / wait kernel -------------------------------------------
+ * Replaces kernel_wait_flag<<<1,1,0,stream>>>(expect, counter), src/wait.cuh:5-9:
+ * spins (s_sleep between agent-scope acquire polls) until *counter == expect,
+ * then resets it to 0.  If the environment variable FO_WAIT_MAX_POLLS is set
+ * to a positive number when the library is first used, this wait (and the one
+ * inside fo_wait_reduce_groups) gives up after that many polls -- a debugging
+ * aid against a hung GPU; unset, the wait is unbounded like the reference's. */
+int fo_wait(int expect, int32_t *counter, fo_stream_t stream);
+
+/* Same, but gives up after max_polls polls (0 = unbounded) and then writes 1
+ * to *status (device int32, may be NULL) without touching the counter; on
+ * success *status is left unchanged.  No counterpart in the reference (its
+ * waiter spins forever); exists so that failure handling can be tested
+ * without hanging a GPU. */
+int fo_wait_bounded(int expect, int32_t *counter, int64_t max_polls, int32_t *status,
+                    fo_stream_t stream);
+
+/* ---- consumer (1-GPU stand-in for the collective) ------------------------
+ * Stands in for ncclAllReduce(C+acc, C+acc, n, half, sum) at
+ * src/overlap_impl.cu:256: acc[i] = round(float(acc[i]) + float(src[i])),
+ * i < nelem; nelem % 8 == 0, 16-byte aligned pointers. */
+int fo_consumer_reduce(int dtype, const void *src, void *acc, int64_t nelem, fo_stream_t stream);
+
+/* Stands in for ncclReduceScatter(C+acc, D+acc/W, n/W) at
+ * src/overlap_impl.cu:312-313 with all W ranks emulated on one GPU: the group
+ * src[0:nelem] holds W equal chunks; chunk q is accumulated into
+ * acc + q*seg_stride (elements).  (nelem/W) % 8 == 0. */
+int fo_consumer_reduce_rs(int dtype, const void *src, void *acc, int64_t nelem, int W,
+                          int64_t seg_stride, fo_stream_t stream);
+
+/* One launch that does, for every group i in order, what the host loop of
+ * src/overlap_impl.cu:250-258 enqueues as 2*G launches: wait until
+ * MM[i] == cseg[i], reset MM[i] to 0, then accumulate the group's contiguous
+ * range of C into ACC (W == 1) or its W chunks into ACC + q*seg_stride at
+ * offset acc/W (W > 1).  ACC == NULL: wait/reset only.  tile_elems = BM*BN.
+ * The counters are reset by the last workgroup to leave instead of per group.
+ * workspace: device int32[2], zero before the first use; the kernel leaves
+ * word 0 zero and sets word 1 only if a bounded poll gave up (see
+ * FO_WAIT_MAX_POLLS below).  nblocks <= 0 picks a default. */
+int fo_wait_reduce_groups(int dtype, const void *C, void *ACC, int32_t *MM,
+                          const int32_t *cseg_dev, int G, int64_t tile_elems, int W,
+                          int64_t seg_stride, int32_t *workspace, int nblocks,
+                          fo_stream_t stream);
+
+/* ---- RMSNorm ----------------------------------------------------------
+ * Replaces reorder_rmsnorm(X, RX, RW, BM, BN, rldn, RA), src/rmsnorm/rmsnorm.h:6-8,
+ * src/rmsnorm/rmsnorm.cu:14-30, kernel src/rmsnorm/rmsnorm.cuh:64-117.
+ * X is the tile-reordered [bs,dim] buffer, Y[bs,dim] row-major output,
+ * Wt[dim].  eps is explicit (the reference hard-codes 1e-5, rmsnorm.cuh:102)
+ * and so is the stream (the reference uses the legacy default stream).
+ * dim % 8 == 0, BN % 8 == 0, bs % BM == 0, dim % BN == 0. */
+int fo_reorder_rmsnorm(int dtype, const void *X, void *Y, const void *Wt, int bs, int dim, int BM,
+                       int BN, int rldn, const int32_t *RA, float eps, fo_stream_t stream);
+
+/* Replaces rmsnorm(X, RX, RW), src/rmsnorm/rmsnorm.cu:32-46, kernel rmsnorm.cuh:14-59. */
+int fo_rmsnorm(int dtype, const void *X, void *Y, const void *Wt, int bs, int dim, float eps,
+               fo_stream_t stream);
+
+/* ---- host orchestration -------------------------------------------------
+ * fo_overlap_t mirrors class OverlapImpl, src/overlap_impl.h:12-43. */
+typedef struct fo_overlap fo_overlap_t;
+
+int fo_overlap_create(fo_overlap_t **out);  /* OverlapImpl(), src/overlap_impl.cu:23-25 */
+int fo_overlap_destroy(fo_overlap_t *h);    /* the reference never releases its streams */
+/* CutlassInit(), src/overlap_impl.cu:31-33: the stream GEMMs are enqueued on. */
+int fo_overlap_set_gemm_stream(fo_overlap_t *h, fo_stream_t gemm_stream);
+/* OverlapInit(), src/overlap_impl.cu:139-141: creates the second (consumer)
+ * stream, non-blocking, default priority. */
+int fo_overlap_init(fo_overlap_t *h);
+/* NcclInit(rank, world, id), src/overlap_impl.cu:50-63: records rank/world; no
+ * communicator is created on one GPU (the reference also keeps comm == NULL
+ * for world == 1). */
+int fo_overlap_set_world(fo_overlap_t *h, int rank, int world);
+/* Accumulation buffer of the stand-in consumer (no counterpart: the reference
+ * reduces across ranks in place).  acc == NULL detaches it.  For W > 1 it is
+ * [W, M/W, N] (seg_stride = M/W*N elements). */
+int fo_overlap_set_accumulator(fo_overlap_t *h, void *acc, int64_t nelem);
+/* fused != 0: use fo_wait_reduce_groups (one launch) instead of 2*G launches. */
+int fo_overlap_set_fused_consumer(fo_overlap_t *h, int fused);
+fo_stream_t fo_overlap_comm_stream(fo_overlap_t *h);
+
+/* Gemm(A,B,C,Algo), src/overlap_impl.cu:35-48. */
+int fo_overlap_gemm(fo_overlap_t *h, int dtype, int M, int N, int K, const void *A, const void *B,
+                    void *C, int algo);
+/* GemmAllReduceOverlap(...), src/overlap_impl.cu:214-264: signal GEMM on the
+ * GEMM stream; per group {wait, consume} on the consumer stream; event join
+ * consumer -> GEMM stream.  cseg_host[G] is host memory. */
+int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int N, int K, const void *A,
+                              const void *B, void *C, int32_t *MM, const int32_t *RA, int TM,
+                              int TN, int rLDN, const int32_t *cseg_host,
+                              const int32_t *cseg_dev, int G, int algo, int monitor);
+/* GemmReduceScatterOverlap(...), src/overlap_impl.cu:266-321.  D[M/W, N]
+ * receives this rank's chunk of every group at offset acc/W (sum over the one
+ * rank present); with an accumulator attached all W chunks are accumulated. */
+int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, int N, int K, const void *A,
+                                  const void *B, void *C, void *D, int32_t *MM, const int32_t *RA,
+                                  const int32_t *RE, int TM, int TN, int rLDN,
+                                  const int32_t *cseg_host, const int32_t *cseg_dev, int G,
+                                  int algo, int monitor);
+/* GemmAllReduce(A,B,C,Algo), src/overlap_impl.cu:65-81: plain GEMM then the
+ * whole-C consumer on the same stream (the non-overlapped comparator). */
+int fo_overlap_gemm_allreduce_serial(fo_overlap_t *h, int dtype, int M, int N, int K,
+                                     const void *A, const void *B, void *C, int algo);
+/* SegAllReduce(C, cSEG_CPU, SegNum), src/overlap_impl.cu:153-167: consumer over
+ * SegNum consecutive segments of M*N/SegNum*cSeg[s] elements, on the GEMM
+ * stream.  G = length of cseg_host (>= seg_num). */
+int fo_overlap_seg_allreduce(fo_overlap_t *h, int dtype, void *C, int64_t MN,
+                             const int32_t *cseg_host, int G, int seg_num);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASHOVERLAP_H */

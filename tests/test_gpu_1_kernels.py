@@ -1,0 +1,271 @@
+"""GPU parity tests of the individual kernels, called through the C ABI (ctypes)
+and checked against the CPU checker on the same seeded inputs.
+
+Tolerances: integer results (permutation, counts, stamps, addresses) and the
+consumer are bit-exact; GEMM and RMSNorm values are compared against the
+fp32-accumulating checker with max rel err <= 1e-2 (and, tighter, within a
+couple of 16-bit ulps, since both sides accumulate in fp32 and round once)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import BF16, F16, TORCH_DTYPE, bits_of, from_bits, max_rel_err, seeded, ulp_diff_ok
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-2  # north-star tolerance for GEMM and RMSNorm values
+
+
+def _algo(fo, bm, bn, swizzle=1):
+    return fo._capi.find_algo(bm, bn, swizzle=swizzle)
+
+
+# ---------------------------------------------------------------- plain GEMM
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("bm,bn,M,N,K", [(128, 128, 256, 384, 192), (128, 256, 256, 512, 128),
+                                         (256, 128, 512, 256, 64), (128, 128, 1024, 1024, 1024)])
+def test_gemm_matches_checker(fo, oracle, dtype, bm, bn, M, N, K):
+    A, Ab = seeded((M, K), dtype, 1)
+    B, Bb = seeded((N, K), dtype, 2, scale=K ** -0.5)
+    C = torch.empty(M, N, device="cuda", dtype=TORCH_DTYPE[dtype])
+    fo.ops.gemm(A, B, C, _algo(fo, bm, bn))
+    torch.cuda.synchronize()
+    ref_bits, _ = oracle.gemm_signal(dtype, Ab, Bb, bm, bn)
+    ref = torch.from_numpy(oracle.from_bits(ref_bits, dtype))
+    assert max_rel_err(C.float().cpu(), ref) <= REL_TOL
+    assert ulp_diff_ok(bits_of(C), ref_bits, dtype, max_ulp=1, frac=0.999)
+
+
+def test_gemm_exact_special_cases(fo):
+    # all ones: every C == K exactly (the reference's own AR test input, correctness_ar.py:24-25)
+    M, N, K = 256, 256, 512
+    A = torch.ones(M, K, device="cuda", dtype=torch.float16)
+    B = torch.ones(N, K, device="cuda", dtype=torch.float16)
+    C = torch.zeros(M, N, device="cuda", dtype=torch.float16)
+    fo.ops.gemm(A, B, C, _algo(fo, 128, 128))
+    assert (C == K).all()
+    # identity weight: C == A bit for bit; catches transposed or mis-indexed operands
+    A, _ = seeded((256, 256), F16, 3)
+    eye = torch.eye(256, device="cuda", dtype=torch.float16)
+    fo.ops.gemm(A, eye, C, _algo(fo, 128, 128))
+    assert torch.equal(C, A)
+    # a one-hot row of B selects a column of A
+    B = torch.zeros(256, 256, device="cuda", dtype=torch.float16)
+    B[5, 77] = 1.0
+    fo.ops.gemm(A, B, C, _algo(fo, 128, 128))
+    assert torch.equal(C[:, 5], A[:, 77]) and C[:, :5].abs().sum() == 0
+
+
+# ---------------------------------------------------------------- signal / scatter GEMM
+def _signal_case(fo, oracle, dtype, bm, bn, M, N, K, cseg, rldn=1, W=0, monitor=False, swizzle=1, seed=4):
+    algo = _algo(fo, bm, bn, swizzle)
+    TM, TN = M // bm, N // bn
+    T = TM * TN
+    rng = np.random.default_rng(seed)
+    hint = rng.permutation(T)[: max(1, T // 2)].tolist()
+    RA = (torch.arange(T, dtype=torch.int32) if monitor else
+          fo.layout.reorder_indices(T, hint, device="cpu")).reshape(TM, TN).cuda()
+    A, Ab = seeded((M, K), dtype, seed + 1)
+    B, Bb = seeded((N, K), dtype, seed + 2, scale=K ** -0.5)
+    plain = torch.empty(M, N, device="cuda", dtype=TORCH_DTYPE[dtype])
+    fo.ops.gemm(A, B, plain, algo)
+    Cp = torch.full((M * N,), float("nan"), device="cuda", dtype=TORCH_DTYPE[dtype])
+    MM = torch.zeros(fo.layout.counter_size(len(cseg), TM, TN, monitor) + 8, dtype=torch.int32, device="cuda")
+    cseg_gpu = torch.tensor(cseg, dtype=torch.int32, device="cuda")
+    RE = fo.layout.generate_row_mapping(M, N, bm, bn, cseg, W, device="cuda") if W else None
+    fo.ops.gemm_signal(A, B, Cp, MM, RA, cseg_gpu, algo, rLDN=rldn, monitor=monitor, RE=RE)
+    torch.cuda.synchronize()
+    ra_np = RA.cpu().numpy().reshape(-1)
+    re_np = None if RE is None else RE.cpu().numpy()
+    # (1) permutation bit-exact: un-permuting with the checker's inverse map gives the plain GEMM
+    back = oracle.unpermute(bits_of(Cp), M, N, bm, bn, ra_np, rLDN=rldn, RE=re_np)
+    assert (back == bits_of(plain)).all()
+    # (2) the package's own torch inverse agrees
+    assert torch.equal(fo.layout.unpermute(Cp, M, N, bm, bn, RA, rLDN=rldn, RE=RE), plain)
+    # (3) every element was written exactly once (no NaN filler left)
+    assert not torch.isnan(Cp).any()
+    # (4) signal counts bit-exact
+    mm = MM.cpu().numpy()
+    if not monitor:
+        assert mm[:len(cseg)].tolist() == list(cseg)
+        assert (mm[len(cseg):] == 0).all()
+    # (5) values against the checker's own reordered buffer
+    ref_bits, ref_mm = oracle.gemm_signal(dtype, Ab, Bb, bm, bn, RA=ra_np, cseg=cseg, rLDN=rldn, RE=re_np)
+    assert ulp_diff_ok(bits_of(Cp), ref_bits, dtype, max_ulp=1, frac=0.999)
+    assert max_rel_err(Cp.float().cpu(), torch.from_numpy(oracle.from_bits(ref_bits, dtype))) <= REL_TOL
+    return mm, T, TN
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+def test_signal_gemm_reorder_and_counts(fo, oracle, dtype):
+    _signal_case(fo, oracle, dtype, 128, 128, 512, 512, 128, [4, 4, 4, 4])
+    _signal_case(fo, oracle, dtype, 128, 128, 512, 512, 128, [1, 15])
+    _signal_case(fo, oracle, dtype, 128, 256, 512, 1024, 64, [5, 3, 8], swizzle=4)
+    _signal_case(fo, oracle, dtype, 256, 128, 1024, 512, 64, [16], swizzle=8)
+
+
+def test_signal_gemm_many_groups_and_rldn(fo, oracle):
+    # more groups than tile columns (the reference under-allocates MM here, test/test.py:94)
+    _signal_case(fo, oracle, F16, 128, 128, 1024, 512, 64, [1] * 32)
+    # 70 groups: the group lookup needs more than one 64-wide scan step
+    _signal_case(fo, oracle, F16, 128, 128, 1280, 1024, 64, [1] * 60 + [2] * 10)
+    # rLDN > 1: the reshaped output is rLDN tiles wide
+    _signal_case(fo, oracle, F16, 128, 128, 512, 512, 64, [8, 8], rldn=2)
+    _signal_case(fo, oracle, F16, 128, 128, 512, 512, 64, [16], rldn=4)
+
+
+def test_scatter_gemm_row_map(fo, oracle):
+    _signal_case(fo, oracle, F16, 128, 128, 512, 512, 64, [4, 4, 8], W=4)
+    _signal_case(fo, oracle, BF16, 128, 128, 512, 256, 128, [3, 5], W=8)
+
+
+def test_monitor_stamps(fo, oracle):
+    mm, T, TN = _signal_case(fo, oracle, F16, 128, 128, 1024, 1024, 64, [16, 16, 16, 16], monitor=True)
+    assert mm[:4].tolist() == [16, 16, 16, 16]
+    assert mm[TN - 1] == T
+    assert sorted(mm[TN:TN + T].tolist()) == list(range(T))
+
+
+# ---------------------------------------------------------------- wait
+def test_wait_bounded_gives_up_and_flags(fo):
+    MM = torch.tensor([3, 0], dtype=torch.int32, device="cuda")
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    fo.ops.wait_bounded(4, MM, 0, 2000, status)          # 3 != 4 forever: must give up
+    torch.cuda.synchronize()
+    assert status.item() == 1 and MM[0].item() == 3       # counter untouched
+    status.zero_()
+    fo.ops.wait_bounded(3, MM, 0, 2000, status)          # already equal: released and reset
+    torch.cuda.synchronize()
+    assert status.item() == 0 and MM[0].item() == 0
+
+
+def test_wait_released_by_second_stream(fo):
+    MM = torch.zeros(4, dtype=torch.int32, device="cuda")
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    done = torch.zeros(1, dtype=torch.int32, device="cuda")
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s1):
+        # bounded (about a minute) so a broken signal path cannot hang the GPU
+        fo.ops.wait_bounded(5, MM, 2, 40_000_000, status, stream=s1)
+        done.add_(1)                                     # ordered after the wait on s1
+    with torch.cuda.stream(s2):
+        for _ in range(5):
+            MM[2:3].add_(1)
+    torch.cuda.synchronize()
+    assert status.item() == 0 and done.item() == 1
+    assert MM.tolist() == [0, 0, 0, 0]                   # reset by the CAS
+
+
+# ---------------------------------------------------------------- consumer
+@pytest.mark.parametrize("dtype", [F16, BF16])
+def test_consumer_bit_exact(fo, oracle, dtype):
+    n = 1 << 18
+    src, sb = seeded((n,), dtype, 20)
+    acc, ab = seeded((n,), dtype, 21, scale=3.0)
+    ref = ab.copy()
+    for _ in range(3):
+        fo.ops.consumer_reduce(src, acc)
+        oracle.consumer_reduce(dtype, sb, ref)
+    torch.cuda.synchronize()
+    assert (bits_of(acc) == ref).all()
+    # closed form on a zeroed accumulator: k calls give k * src when k * src is exact
+    acc.zero_()
+    fo.ops.consumer_reduce(src, acc)
+    fo.ops.consumer_reduce(src, acc)
+    assert torch.equal(acc, (src.float() * 2).to(src.dtype))
+
+
+def test_consumer_reduce_scatter_layout(fo, oracle):
+    W, chunk = 4, 4096
+    src, sb = seeded((W * chunk,), F16, 22)
+    seg = 3 * chunk
+    acc = torch.zeros(W * seg, device="cuda", dtype=torch.float16)
+    fo.ops.consumer_reduce_rs(src, acc[chunk:], W, seg)     # offset inside every segment
+    torch.cuda.synchronize()
+    a = acc.view(W, seg)
+    for q in range(W):
+        assert torch.equal(a[q, chunk:2 * chunk], src[q * chunk:(q + 1) * chunk])
+        assert a[q, :chunk].abs().sum() == 0 and a[q, 2 * chunk:].abs().sum() == 0
+
+
+# ---------------------------------------------------------------- RMSNorm
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("bs,dim", [(64, 256), (32, 4096), (16, 8192), (8, 1000 * 8), (4, 16384)])
+def test_rmsnorm_matches_checker(fo, oracle, dtype, bs, dim):
+    X, Xb = seeded((bs, dim), dtype, 30, scale=2.0)
+    g = torch.Generator().manual_seed(31)
+    W16 = (1 + 0.01 * torch.randn(dim, generator=g)).to(TORCH_DTYPE[dtype])
+    Y = torch.empty_like(X)
+    fo.ops.rmsnorm(X, Y, W16.cuda(), eps=1e-6)
+    torch.cuda.synchronize()
+    ref_bits = oracle.rmsnorm(dtype, Xb, bits_of(W16), bs, dim, eps=1e-6)
+    ref = torch.from_numpy(oracle.from_bits(ref_bits, dtype)).reshape(bs, dim)
+    assert max_rel_err(Y.float().cpu(), ref) <= REL_TOL
+    assert ulp_diff_ok(bits_of(Y), ref_bits, dtype, max_ulp=2, frac=0.99)
+    # textbook formula of example/RMSNorm.py:13-18 on the GPU
+    xf = X.float()
+    tb = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-6)).type_as(X) * W16.cuda()
+    assert max_rel_err(Y.float(), tb.float()) <= REL_TOL
+
+
+def test_rmsnorm_constant_row_closed_form(fo):
+    dim, c, eps = 512, 3.0, 1e-5
+    X = torch.full((4, dim), c, device="cuda", dtype=torch.float16)
+    Wt = torch.linspace(0.5, 1.5, dim).to(torch.float16).cuda()
+    Y = torch.empty_like(X)
+    fo.ops.rmsnorm(X, Y, Wt, eps=eps)
+    xn = torch.tensor(c / np.sqrt(c * c + eps), dtype=torch.float32).to(torch.float16)
+    expect = (xn.float() * Wt.float().cpu()).to(torch.float16)
+    got = Y[0].cpu()
+    assert ((got.view(torch.int16).int() - expect.view(torch.int16).int()).abs() <= 1).all()
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+def test_reorder_rmsnorm_undoes_the_permutation(fo, oracle, dtype):
+    for (bm, bn, M, N, rldn) in [(128, 128, 256, 1024, 1), (128, 256, 256, 4096, 1), (64, 128, 256, 512, 2),
+                                 (16, 128, 64, 8192, 1)]:
+        TM, TN = M // bm, N // bn
+        T = TM * TN
+        rng = np.random.default_rng(40)
+        ra = rng.permutation(T).astype(np.int32)
+        plain, pb = seeded((M, N), dtype, 41, scale=1.5)
+        _, wb = seeded((N,), dtype, 42)
+        Wt = from_bits(wb, dtype)
+        # build the reordered buffer on the host with the checker-independent brute force of the address map
+        Cp = np.empty(M * N, dtype=np.uint16)
+        ldp = rldn * bn
+        view = Cp.reshape(-1, ldp)
+        for tm in range(TM):
+            for tn in range(TN):
+                r = ra[tm * TN + tn]
+                view[(r // rldn) * bm:(r // rldn + 1) * bm, (r % rldn) * bn:(r % rldn + 1) * bn] = \
+                    pb[tm * bm:(tm + 1) * bm, tn * bn:(tn + 1) * bn]
+        X = from_bits(Cp, dtype).reshape(M, N)
+        RA = torch.from_numpy(ra).cuda()
+        Y = torch.empty(M, N, device="cuda", dtype=TORCH_DTYPE[dtype])
+        Yp = torch.empty_like(Y)
+        fo.ops.reorder_rmsnorm(X, Y, Wt, bm, bn, rldn, RA, eps=1e-6)
+        fo.ops.rmsnorm(plain, Yp, Wt, eps=1e-6)
+        torch.cuda.synchronize()
+        assert torch.equal(Y, Yp)                       # the gather is exact: same bits as plain RMSNorm
+        ref_bits = oracle.reorder_rmsnorm(dtype, Cp, wb, M, N, bm, bn, rldn, ra, eps=1e-6)
+        assert ulp_diff_ok(bits_of(Y), ref_bits, dtype, max_ulp=2, frac=0.99)
+        ref = torch.from_numpy(oracle.from_bits(ref_bits, dtype)).reshape(M, N)
+        assert max_rel_err(Y.float().cpu(), ref) <= REL_TOL
+
+
+def test_error_codes_on_gpu(fo):
+    A = torch.zeros(128, 64, device="cuda", dtype=torch.float16)
+    C = torch.zeros(128, 128, device="cuda", dtype=torch.float16)
+    with pytest.raises(fo.FlashOverlapError) as e:
+        fo.ops.gemm(A, torch.zeros(100, 64, device="cuda", dtype=torch.float16),
+                    torch.zeros(128, 100, device="cuda", dtype=torch.float16), 0)
+    assert e.value.code == -2
+    with pytest.raises(fo.FlashOverlapError) as e:
+        fo.ops.gemm(A, A, C, 500)
+    assert e.value.code == -3
+    with pytest.raises(TypeError):
+        fo.ops.gemm(A.float(), A.float(), C.float(), 0)

@@ -1,0 +1,307 @@
+"""GPU parity tests of the overlapped path: signal GEMM on one stream, per-group
+wait + consumer on the second, reorder+RMSNorm after the join.  Through the C-ABI
+handle (ctypes) and through the drop-in torch.classes / torch.ops boundary; at
+small sizes against the CPU checker, at the BASELINE.json sizes through
+size-independent properties (round trip, exact doubling, counters back to zero)
+plus sampled rows against an fp32 CPU product."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import BF16, F16, TORCH_DTYPE, bits_of, max_rel_err, seeded, ulp_diff_ok
+
+pytestmark = pytest.mark.gpu
+REL_TOL = 1e-2
+
+
+def _setup(fo, dtype, bm, bn, M, N, K, cseg, swizzle=1, seed=50, hint=None):
+    algo = fo._capi.find_algo(bm, bn, swizzle=swizzle)
+    TM, TN = M // bm, N // bn
+    if hint is None:
+        hint = fo._capi.schedule_order(algo, M, N)     # analytic completion order
+    RA = fo.layout.reorder_indices(TM * TN, hint, device="cuda").reshape(TM, TN)
+    A, Ab = seeded((M, K), dtype, seed)
+    B, Bb = seeded((N, K), dtype, seed + 1, scale=K ** -0.5)
+    MM = torch.zeros(fo.layout.counter_size(len(cseg), TM, TN), dtype=torch.int32, device="cuda")
+    cseg_cpu = torch.tensor(cseg, dtype=torch.int32)
+    return algo, RA, A, B, Ab, Bb, MM, cseg_cpu, cseg_cpu.cuda()
+
+
+@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("dtype", [F16, BF16])
+def test_allreduce_overlap_against_checker(fo, oracle, dtype, fused):
+    bm, bn, M, N, K = 128, 128, 1024, 1024, 256
+    cseg = [16, 16, 8, 24]
+    algo, RA, A, B, Ab, Bb, MM, cs_cpu, cs_gpu = _setup(fo, dtype, bm, bn, M, N, K, cseg)
+    td = TORCH_DTYPE[dtype]
+    Cp = torch.empty(M * N, device="cuda", dtype=td)
+    acc0, acc0_bits = seeded((M * N,), dtype, 60, scale=0.5)
+    ACC = acc0.clone()
+    ov = fo.ops.Overlap()
+    ov.set_fused_consumer(fused)
+    ov.set_accumulator(ACC)
+    ov.gemm_allreduce_overlap(A, B, Cp, MM, RA, 1, cs_cpu, cs_gpu, algo)
+    torch.cuda.synchronize()
+    assert (MM == 0).all()                                   # every wait reset its counter
+    # checker: signal GEMM, then the host schedule (wait + consume per group)
+    ra_np = RA.cpu().numpy().reshape(-1)
+    ref_c, ref_mm = oracle.gemm_signal(dtype, Ab, Bb, bm, bn, RA=ra_np, cseg=cseg)
+    assert ulp_diff_ok(bits_of(Cp), ref_c, dtype, max_ulp=1, frac=0.999)
+    # the consumer is exact given its input: run the checker's schedule on the GPU's own C'
+    mm = np.zeros_like(ref_mm)
+    mm[:len(cseg)] = cseg
+    ref_acc = acc0_bits.copy()
+    assert oracle.host_schedule(dtype, bm * bn, cseg, mm, bits_of(Cp), ACC=ref_acc) == 0
+    assert (bits_of(ACC) == ref_acc).all()
+    # second call on the same handle: counters were clean, ACC accumulates again
+    ov.gemm_allreduce_overlap(A, B, Cp, MM, RA, 1, cs_cpu, cs_gpu, algo)
+    torch.cuda.synchronize()
+    mm[:len(cseg)] = cseg
+    assert oracle.host_schedule(dtype, bm * bn, cseg, mm, bits_of(Cp), ACC=ref_acc) == 0
+    assert (bits_of(ACC) == ref_acc).all() and (MM == 0).all()
+    # serial comparator produces the same C (row-major) and the same kind of accumulation
+    Cs = torch.empty(M, N, device="cuda", dtype=td)
+    ACC.zero_()
+    ov.gemm_allreduce(A, B, Cs, algo)
+    torch.cuda.synchronize()
+    assert torch.equal(fo.layout.unpermute(Cp, M, N, bm, bn, RA), Cs)
+    assert torch.equal(ACC.view(M, N), Cs)
+    ov.close()
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_reducescatter_overlap_segments(fo, oracle, fused):
+    dtype, W, rank = F16, 4, 2
+    bm, bn, M, N, K = 128, 128, 1024, 512, 128
+    cseg = [8, 8, 16]
+    algo, RA, A, B, Ab, Bb, MM, cs_cpu, cs_gpu = _setup(fo, dtype, bm, bn, M, N, K, cseg)
+    RE = fo.layout.generate_row_mapping(M, N, bm, bn, cseg, W, device="cuda")
+    Cp = torch.empty(M * N, device="cuda", dtype=torch.float16)
+    D = torch.zeros(M // W, N, device="cuda", dtype=torch.float16)
+    ACC = torch.zeros(W, M // W, N, device="cuda", dtype=torch.float16)
+    plain = torch.empty(M, N, device="cuda", dtype=torch.float16)
+    ov = fo.ops.Overlap(rank=rank, world=W)
+    ov.set_fused_consumer(fused)
+    ov.set_accumulator(ACC)
+    ov.gemm(A, B, plain, algo)
+    ov.gemm_reducescatter_overlap(A, B, Cp, D, MM, RA, RE, 1, cs_cpu, cs_gpu, algo)
+    torch.cuda.synchronize()
+    assert (MM == 0).all()
+    # segment q, un-permuted with tile (BM/W, BN) and the same RA, is rows q, q+W, ... of the product
+    for q in range(W):
+        seg = fo.layout.unpermute(ACC[q].reshape(-1), M // W, N, bm // W, bn, RA)
+        assert torch.equal(seg, plain[q::W])
+    assert torch.equal(D, ACC[rank])                       # D = this rank's chunk (one rank: sum = copy)
+    # the checker's schedule on the GPU's C' gives the same segments bit for bit
+    mm = np.zeros(MM.numel(), dtype=np.int32)
+    mm[:len(cseg)] = cseg
+    ref = np.zeros(W * (M // W) * N, dtype=np.uint16)
+    assert oracle.host_schedule(dtype, bm * bn, cseg, mm, bits_of(Cp), ACC=ref, W=W,
+                                seg_stride=(M // W) * N) == 0
+    assert (bits_of(ACC).reshape(-1) == ref).all()
+    ov.close()
+
+
+def test_overlap_error_paths(fo):
+    bm, bn, M, N, K = 128, 128, 256, 256, 64
+    algo, RA, A, B, _, _, MM, cs_cpu, cs_gpu = _setup(fo, F16, bm, bn, M, N, K, [2, 2])
+    C = torch.empty(M * N, device="cuda", dtype=torch.float16)
+    ov = fo.ops.Overlap()
+    bad = torch.tensor([2, 1], dtype=torch.int32)           # sum != tile count: rejected before any launch
+    with pytest.raises(fo.FlashOverlapError) as e:
+        ov.gemm_allreduce_overlap(A, B, C, MM, RA, 1, bad, bad.cuda(), algo)
+    assert e.value.code == -5
+    with pytest.raises(fo.FlashOverlapError) as e:          # RA shape does not match the Algo's tile
+        ov.gemm_allreduce_overlap(A, B, C, MM, RA.reshape(1, 4), 1, cs_cpu, cs_gpu, algo)
+    assert e.value.code == -2
+    ov.gemm_allreduce_overlap(A, B, C, MM, RA, 1, cs_cpu, cs_gpu, algo)   # still usable afterwards
+    torch.cuda.synchronize()
+    assert (MM == 0).all()
+    ov.close()
+
+
+# ---------------------------------------------------------------- drop-in boundary (torch.classes / torch.ops)
+def test_dropin_layers_match_reference_semantics(fo):
+    """Shape of example/correctness_ar.py:21-57 on one GPU: baseline linear + RMSNorm
+    against overlap linear + ReorderRMSNorm, allclose(atol=rtol=1e-2)."""
+    from flashoverlap_amd import layers
+    M, N, K = 1024, 1024, 512
+    algo = fo._capi.find_algo(128, 128)
+    hint = fo._capi.schedule_order(algo, M, N)
+    config = {"BM": 128, "BN": 128, "Algo": algo, "hint": hint, "cSeg": [16, 16, 32], "rLDN": 1}
+    layers.load_library()
+    nccl_id = torch.ops.flashoverlap_op.generate_nccl_id()
+    torch.manual_seed(0)
+    for ones in (True, False):
+        base = layers.RowParallelLayer(K, N, "all_reduce")
+        over = layers.OverlapRowParallelLayer(0, 1, K, N, M, config, "all_reduce", nccl_id)
+        if ones:                                            # the reference's input: every C == K
+            x = torch.ones(M, K, device="cuda", dtype=torch.float16)
+            base.weight.data.fill_(1.0)
+        else:
+            x = torch.randn(M, K, device="cuda").half()
+            base.weight.data.mul_(K ** -0.5)
+        over.weight.data.copy_(base.weight.data)
+        norm = layers.RMSNorm(N)
+        rnorm = layers.ReorderRMSNorm(N, M, 128, 128, hint)
+        rnorm.weight.data.copy_(norm.weight.data)
+        with torch.no_grad():
+            ref = norm(base(x))
+            got = rnorm(over(x))
+        torch.cuda.synchronize()
+        assert torch.allclose(got, ref, atol=1e-2, rtol=1e-2)
+        assert (over.counter == 0).all()
+
+
+def test_dropin_reducescatter_layer(fo):
+    """Shape of example/correctness_rs.py:22-71: the baseline sees rows sorted by row % W."""
+    from flashoverlap_amd import layers
+    M, N, K, W, rank = 1024, 512, 256, 4, 1
+    algo = fo._capi.find_algo(128, 128)
+    hint = fo._capi.schedule_order(algo, M, N)
+    config = {"BM": 128, "BN": 128, "Algo": algo, "hint": hint, "cSeg": [8, 24], "rLDN": 1}
+    torch.manual_seed(1)
+    x = torch.randn(M, K, device="cuda").half()
+    base = layers.RowParallelLayer(K, N, "reduce_scatter", rank=rank, world_size=W)
+    base.weight.data.mul_(K ** -0.5)
+    over = layers.OverlapRowParallelLayer(rank, W, K, N, M, config, "reduce_scatter", [0] * 16)
+    over.weight.data.copy_(base.weight.data)
+    norm = layers.RMSNorm(N)
+    rnorm = layers.ReorderRMSNorm(N, M // W, 128 // W, 128, hint)
+    rnorm.weight.data.copy_(norm.weight.data)
+    with torch.no_grad():
+        ref = norm(base(fo.layout.reorder_rows_by_world_size(x, W)))
+        got = rnorm(over(x))
+    torch.cuda.synchronize()
+    assert torch.allclose(got, ref, atol=5e-2, rtol=5e-2)     # the reference's RS tolerance
+    assert torch.allclose(got, ref, atol=1e-2, rtol=1e-2)
+
+
+def test_dropin_class_methods(fo):
+    from flashoverlap_amd import layers
+    layers.load_library()
+    M = N = 256
+    K = 128
+    A = torch.randn(M, K, device="cuda").half()
+    B = torch.randn(N, K, device="cuda").half()
+    C = torch.empty(M, N, device="cuda", dtype=torch.float16)
+    C2 = torch.empty_like(C)
+    ov = torch.classes.flashoverlap_class.OverlapImpl()
+    ov.nccl_init(0, 1, torch.ops.flashoverlap_op.generate_nccl_id())
+    ov.cutlass_init()
+    ov.overlap_init()
+    ov.cutlass_gemm(A, B, C, 0)
+    bl = torch.classes.flashoverlap_class.BaselineImpl()
+    bl.nccl_init(0, 1, [0] * 16)
+    bl.cublas_init()
+    bl.cublas_gemm(A, B, C2)
+    torch.cuda.synchronize()
+    ref = A.float() @ B.float().T
+    assert max_rel_err(C.float(), ref) <= REL_TOL and max_rel_err(C2.float(), ref) <= REL_TOL
+    acc = torch.zeros_like(C)
+    ov.set_accumulator(acc)
+    ov.gemm_allreduce(A, B, C, 0)                         # GEMM, then the whole-C consumer
+    torch.cuda.synchronize()
+    assert torch.equal(acc, C)
+    ov.nccl_allreduce(C)
+    ov.seg_allreduce(C, torch.tensor([1, 1], dtype=torch.int32), 2)   # two segments of M*N/2
+    torch.cuda.synchronize()
+    twice = (C.float() * 2).half()
+    assert torch.equal(acc, (twice.float() + C.float()).half())
+    with pytest.raises(RuntimeError):                     # 1/2 + 3/2 of M*N overruns C
+        ov.seg_allreduce(C, torch.tensor([1, 3], dtype=torch.int32), 2)
+    D = torch.empty(M // 2, N, device="cuda", dtype=torch.float16)
+    ov2 = torch.classes.flashoverlap_class.OverlapImpl()
+    ov2.nccl_init(1, 2, [0] * 16)
+    ov2.cutlass_init()
+    ov2.gemm_reducescatter(A, B, C, D, 0)                 # whole-C reduce-scatter: rank 1's half
+    torch.cuda.synchronize()
+    assert torch.equal(D, C[M // 2:])
+
+
+# ---------------------------------------------------------------- BASELINE.json configurations at full size
+def _full_size_case(fo, dtype, bm, bn, M, N, K, cseg, swizzle, W=0, a_outliers=False, dist="normal", seed=70):
+    algo = fo._capi.find_algo(bm, bn, swizzle=swizzle)
+    TM, TN = M // bm, N // bn
+    hint = fo._capi.schedule_order(algo, M, N)
+    RA = fo.layout.reorder_indices(TM * TN, hint, device="cuda").reshape(TM, TN)
+    td = TORCH_DTYPE[dtype]
+    g = torch.Generator().manual_seed(seed)
+    if dist == "uniform":
+        Af = (torch.rand(M, K, generator=g) * 2 - 1) * K ** -0.5
+        Bf = (torch.rand(N, K, generator=g) * 2 - 1) * K ** -0.5
+    else:
+        Af = torch.randn(M, K, generator=g)
+        Bf = torch.randn(N, K, generator=g) * K ** -0.5
+    if a_outliers:                                         # 5% outlier columns scaled x8
+        cols = torch.randperm(K, generator=g)[: int(np.ceil(0.05 * K))]
+        Af[:, cols] *= 8
+    A16, B16 = Af.to(td), Bf.to(td)
+    A, B = A16.cuda(), B16.cuda()
+    MM = torch.zeros(fo.layout.counter_size(len(cseg), TM, TN), dtype=torch.int32, device="cuda")
+    cs_cpu = torch.tensor(cseg, dtype=torch.int32)
+    cs_gpu = cs_cpu.cuda()
+    plain = torch.empty(M, N, device="cuda", dtype=td)
+    Cp = torch.empty(M * N, device="cuda", dtype=td)
+    ov = fo.ops.Overlap(rank=0, world=max(W, 1))
+    ACC = torch.zeros(M * N, device="cuda", dtype=td)
+    ov.set_accumulator(ACC)
+    ov.gemm(A, B, plain, algo)
+    RE = None
+    if W:
+        RE = fo.layout.generate_row_mapping(M, N, bm, bn, cseg, W, device="cuda")
+        D = torch.empty(M // W, N, device="cuda", dtype=td)
+        for _ in range(2):
+            ov.gemm_reducescatter_overlap(A, B, Cp, D, MM, RA, RE, 1, cs_cpu, cs_gpu, algo)
+    else:
+        for _ in range(2):
+            ov.gemm_allreduce_overlap(A, B, Cp, MM, RA, 1, cs_cpu, cs_gpu, algo)
+    torch.cuda.synchronize()
+    assert (MM == 0).all()                                                  # signal counts consumed exactly
+    assert torch.equal(fo.layout.unpermute(Cp, M, N, bm, bn, RA, RE=RE), plain)   # permutation bit-exact
+    if W:
+        seg = ACC.view(W, M // W, N)
+        for q in (0, W - 1):
+            un = fo.layout.unpermute(seg[q].reshape(-1), M // W, N, bm // W, bn, RA)
+            assert torch.equal(un, (plain[q::W].float() * 2).to(td))        # two calls: exact doubling
+    else:
+        assert torch.equal(ACC, (Cp.float() * 2).to(td))
+    # sampled rows against an fp32 CPU product of the same 16-bit inputs
+    rows = torch.randperm(M, generator=g)[:48]
+    ref = A16[rows].float() @ B16.float().T
+    assert max_rel_err(plain[rows.cuda()].float().cpu(), ref) <= REL_TOL
+    # reorder+RMSNorm over the overlapped output equals RMSNorm of the plain product
+    gamma = (1 + 0.01 * torch.randn(N, generator=g)).to(td).cuda()
+    if W:
+        X, bs, tile_m = ACC.view(W, M // W, N)[0].contiguous(), M // W, bm // W
+        want_src = (plain[0::W].float() * 2).to(td)
+    else:
+        X, bs, tile_m = Cp.view(M, N), M, bm
+        want_src = plain
+    Y = torch.empty(bs, N, device="cuda", dtype=td)
+    Yref = torch.empty_like(Y)
+    fo.ops.reorder_rmsnorm(X, Y, gamma, tile_m, bn, 1, RA, eps=1e-6)
+    fo.ops.rmsnorm(want_src.contiguous(), Yref, gamma, eps=1e-6)
+    torch.cuda.synchronize()
+    assert torch.equal(Y, Yref)
+    xr = want_src[:32].float()
+    tb = (xr * torch.rsqrt(xr.pow(2).mean(-1, keepdim=True) + 1e-6)).to(td) * gamma
+    assert max_rel_err(Y[:32].float(), tb.float()) <= REL_TOL
+    ov.close()
+
+
+def test_config2_row_parallel_k_slice(fo):
+    _full_size_case(fo, F16, 128, 128, 4096, 4096, 512, [4] * 256, swizzle=4)
+
+
+def test_config3_mlp_down_projection_bf16(fo):
+    _full_size_case(fo, BF16, 256, 128, 8192, 8192, 3584, [512, 512, 1024], swizzle=4, a_outliers=True)
+
+
+def test_config4_reduce_scatter_layout(fo):
+    _full_size_case(fo, F16, 128, 128, 8192, 4096, 4096, [512, 512, 512, 512], swizzle=4, W=8)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+def test_config5_large_square(fo, dtype):
+    _full_size_case(fo, dtype, 128, 256, 8192, 8192, 8192, [256] * 8, swizzle=4, dist="uniform")

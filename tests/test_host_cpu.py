@@ -1,0 +1,152 @@
+"""CPU-side checks of the product: the C-ABI library loads and exports every
+symbol the header declares, validates arguments before touching a GPU, owns the
+reference's Algo table and a consistent tile schedule; the Python host logic
+(latency model, searches, config JSON) agrees with the CPU checker."""
+import ctypes
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from flashoverlap_amd import _capi, config, layout, tune
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _header_symbols():
+    text = open(os.path.join(ROOT, "include", "flashoverlap.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fo_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    L = ctypes.CDLL(_capi.KERNEL_LIB)
+    names = _header_symbols()
+    assert len(names) >= 25
+    for n in names:
+        assert hasattr(L, n), f"libfo_kernels.so does not export {n}"
+    assert set(names) == set(_capi.SIGNATURES), "ctypes table and header disagree"
+
+
+def test_shim_registers_reference_names():
+    from flashoverlap_amd import layers
+    layers.load_library()
+    ov = torch.classes.flashoverlap_class.OverlapImpl()
+    for m in ["nccl_init", "cutlass_init", "overlap_init", "cutlass_gemm", "gemm_allreduce_overlap",
+              "gemm_reducescatter_overlap", "gemm_allreduce", "gemm_reducescatter", "gemm_all2all",
+              "nccl_allreduce", "nccl_reducescatter", "nccl_all2all", "seg_allreduce"]:
+        assert hasattr(ov, m), m
+    bl = torch.classes.flashoverlap_class.BaselineImpl()
+    for m in ["nccl_init", "cublas_init", "cublas_gemm", "gemm_allreduce", "gemm_reducescatter",
+              "gemm_all2all", "nccl_allreduce", "nccl_reducescatter", "nccl_all2all"]:
+        assert hasattr(bl, m), m
+    ident = torch.ops.flashoverlap_op.generate_nccl_id()
+    assert len(ident) == 16                       # 128 bytes as int64, src/nccl_utils.cu:7-14
+    assert hasattr(torch.ops.flashoverlap_op, "reorder_rmsnorm")
+    # dtype errors surface as exceptions, as data_ptr<at::Half>() does in the reference
+    x = torch.zeros(4, 8)
+    with pytest.raises(RuntimeError):
+        torch.ops.flashoverlap_op.reorder_rmsnorm(x, x, x[0], 4, 8, 1, torch.zeros(1, 1, dtype=torch.int32))
+
+
+def test_algo_table_matches_reference_rows():
+    golden = json.load(open(os.path.join(GOLDEN, "algo_table.json")))["rows"]
+    assert [list(r) for r in _capi.algo_table()] == golden
+    assert _capi.algo_tile(0) == (128, 128) and _capi.algo_tile(54) == (128, 256)
+    assert _capi.algo_tile(78) == (256, 128)
+    assert _capi.find_algo(128, 256, swizzle=4) == 57
+
+
+def test_argument_validation_without_gpu():
+    L = _capi.lib()
+    null = ctypes.c_void_p()
+    one = ctypes.c_void_p(16)  # never dereferenced: validation fails first
+    assert L.fo_gemm(0, 128, 128, 64, null, one, one, 0, null) == -1           # null A
+    assert L.fo_gemm(0, 100, 128, 64, one, one, one, 0, null) == -2            # M % 128
+    assert L.fo_gemm(0, 128, 128, 70, one, one, one, 0, null) == -2            # K % 64
+    assert L.fo_gemm(0, 128, 128, 64, one, one, one, 102, null) == -3          # Algo range
+    assert L.fo_gemm(7, 128, 128, 64, one, one, one, 0, null) == -4            # dtype
+    assert L.fo_gemm_signal(0, 128, 128, 64, 1, one, 0, one, one, one, one, one, 0, 0, null) == -5
+    # monitor mode keeps its order counter at MM[TN-1]: needs G <= TN-1
+    assert L.fo_gemm_signal(0, 128, 128, 64, 1, one, 1, one, one, one, one, one, 1, 0, null) == -5
+    assert L.fo_wait(1, null, null) == -1
+    assert L.fo_consumer_reduce(0, one, one, 12, null) == -2                   # nelem % 8
+    assert L.fo_reorder_rmsnorm(0, one, one, one, 8, 100, 4, 50, 1, one, 1e-5, null) == -2
+    assert L.fo_overlap_gemm(null, 0, 128, 128, 64, one, one, one, 0) == -1
+    h = ctypes.c_void_p()
+    assert L.fo_overlap_create(ctypes.byref(h)) == 0
+    assert L.fo_overlap_gemm(h, 0, 128, 128, 64, one, one, one, 0) == -6       # before cutlass_init
+    assert L.fo_overlap_set_world(h, 2, 2) == -1
+    assert L.fo_overlap_set_world(h, 1, 8) == 0
+    assert L.fo_overlap_destroy(h) == 0
+    assert b"Algo" in L.fo_error_string(-3)
+
+
+@pytest.mark.parametrize("algo,M,N", [(0, 1024, 1024), (3, 4096, 4096), (57, 8192, 8192),
+                                       (80, 8192, 8192), (5, 384, 640), (0, 128, 128)])
+def test_schedule_order_is_a_permutation_with_local_waves(algo, M, N):
+    order = _capi.schedule_order(algo, M, N)
+    bm, bn = _capi.algo_tile(algo)
+    TM, TN = M // bm, N // bn
+    assert sorted(order) == list(range(TM * TN))
+    if TM * TN >= 256 and (TM * TN) % 8 == 0:
+        # one wave of 256 workgroups: 32 consecutive raster positions per XCD, so each
+        # XCD's share of the wave spans few distinct tile rows/columns
+        wave = order[:256]
+        for x in range(8):
+            mine = wave[x::8]
+            rows = {t // TN for t in mine}
+            cols = {t % TN for t in mine}
+            assert len(rows) * len(cols) <= 64
+
+
+def test_latency_model_and_search_agree_with_checker(oracle):
+    curve = np.array([[2.0 ** (20 + 0.25 * i), 0.5 + 0.1 * i] for i in range(36)])
+    M = N = 8192
+    tiles, wave = 2048, 256
+    for gp in ([2048], [256] * 8, [512, 512, 1024], [256, 1792], [1000, 1048]):
+        a = tune.predict_latency(M, N, 0.7, curve, gp, tiles, wave, 256)
+        b = oracle.predict_latency(M, N, 0.7, curve[:, 0], curve[:, 1], gp, tiles, wave, 256, 6.0)
+        assert a == pytest.approx(b, rel=1e-12)
+    assert tune.integer_partitions(4) == oracle.compositions(4)
+    assert tune.groups_to_cseg([1, 2, 1], 256, 1000) == [256, 512, 232]
+    best, dur = tune.predictive_search(M, N, 0.7, curve, tiles, wave)
+    assert sum(best) == tiles and all(c % wave == 0 for c in best[:-1])
+    # exhaustive check of the argmin over the same candidate set
+    cands = [tune.groups_to_cseg(gp, wave, tiles) for gp in tune.integer_partitions(8)
+             if not (len(gp) > 5 and gp[0] > 2)]
+    assert dur == pytest.approx(min(tune.predict_latency(M, N, 0.7, curve, c, tiles, wave) for c in cands))
+
+
+def test_config_json_two_stage_round_trip(tmp_path):
+    assert config.gpu_tag("NVIDIA A800-SXM4-80GB") == "a800"      # the reference's slicing rule
+    assert config.gpu_tag("AMD Instinct MI355X") == "tinc"
+    d = str(tmp_path)
+    p = config.save_gemm_candidates(4096, 4096, 512, [128, 128], [128, 256], [0.1, 0.2], [3, 57],
+                                    gpu="tinc", directory=d)
+    assert os.path.basename(p) == "m4096n4096k512_tinc.json"
+    assert config.load_gemm_candidates(4096, 4096, 512, gpu="tinc", directory=d) == \
+        ([128, 128], [128, 256], [0.1, 0.2], [3, 57])
+    with pytest.raises(ValueError):
+        config.load_solution(4096, 4096, 512, gpu="tinc", directory=d)
+    config.save_solution(4096, 4096, 512, 128, 128, 0.1, 3, [1, 0], [512, 512], gpu="tinc", directory=d)
+    sol = config.load_solution(4096, 4096, 512, gpu="tinc", directory=d)
+    assert sol == {"BM": 128, "BN": 128, "dur": 0.1, "Algo": 3, "hint": [1, 0], "cSeg": [512, 512],
+                   "rLDN": 1}
+
+
+def test_layout_matches_checker_on_random_cases(oracle):
+    rng = np.random.default_rng(3)
+    for _ in range(10):
+        BM, BN, W = int(rng.choice([4, 8])), int(rng.choice([8, 16])), int(rng.choice([1, 2, 4]))
+        TM, TN = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        T = TM * TN
+        cuts = sorted(rng.choice(np.arange(1, T), size=min(T - 1, int(rng.integers(0, 4))), replace=False).tolist()) if T > 1 else []
+        cseg = [b - a for a, b in zip([0] + cuts, cuts + [T])]
+        got = layout.generate_row_mapping(TM * BM, TN * BN, BM, BN, cseg, W, device="cpu")
+        assert got.tolist() == oracle.row_mapping(TM * BM, TN * BN, BM, BN, cseg, W).tolist()
+        assert layout.tile_groups(cseg).tolist() == [oracle.tile_group(cseg, r) for r in range(T)]
