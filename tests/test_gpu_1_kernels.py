@@ -11,7 +11,8 @@ import numpy as np
 import pytest
 import torch
 
-from gpu_util import BF16, F16, TORCH_DTYPE, bits_of, from_bits, max_rel_err, seeded, ulp_diff_ok
+from gpu_util import (BF16, F16, TORCH_DTYPE, bits_of, from_bits, max_rel_err, rmsnorm_f64, seeded,
+                      ulp_diff_ok)
 
 pytestmark = pytest.mark.gpu
 
@@ -202,13 +203,11 @@ def test_rmsnorm_matches_checker(fo, oracle, dtype, bs, dim):
     fo.ops.rmsnorm(X, Y, W16.cuda(), eps=1e-6)
     torch.cuda.synchronize()
     ref_bits = oracle.rmsnorm(dtype, Xb, bits_of(W16), bs, dim, eps=1e-6)
-    ref = torch.from_numpy(oracle.from_bits(ref_bits, dtype)).reshape(bs, dim)
-    assert max_rel_err(Y.float().cpu(), ref) <= REL_TOL
     assert ulp_diff_ok(bits_of(Y), ref_bits, dtype, max_ulp=2, frac=0.99)
-    # textbook formula of example/RMSNorm.py:13-18 on the GPU
-    xf = X.float()
-    tb = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-6)).type_as(X) * W16.cuda()
-    assert max_rel_err(Y.float(), tb.float()) <= REL_TOL
+    # 1e-2 against the unrounded formula of example/RMSNorm.py:13-18 (both the GPU and the checker)
+    exact = rmsnorm_f64(X, W16, 1e-6)
+    assert max_rel_err(Y.cpu(), exact) <= REL_TOL
+    assert max_rel_err(torch.from_numpy(oracle.from_bits(ref_bits, dtype)).reshape(bs, dim), exact) <= REL_TOL
 
 
 def test_rmsnorm_constant_row_closed_form(fo):
@@ -253,8 +252,7 @@ def test_reorder_rmsnorm_undoes_the_permutation(fo, oracle, dtype):
         assert torch.equal(Y, Yp)                       # the gather is exact: same bits as plain RMSNorm
         ref_bits = oracle.reorder_rmsnorm(dtype, Cp, wb, M, N, bm, bn, rldn, ra, eps=1e-6)
         assert ulp_diff_ok(bits_of(Y), ref_bits, dtype, max_ulp=2, frac=0.99)
-        ref = torch.from_numpy(oracle.from_bits(ref_bits, dtype)).reshape(M, N)
-        assert max_rel_err(Y.float().cpu(), ref) <= REL_TOL
+        assert max_rel_err(Y.cpu(), rmsnorm_f64(plain, Wt, 1e-6)) <= REL_TOL
 
 
 def test_error_codes_on_gpu(fo):
