@@ -1,0 +1,183 @@
+"""One-GPU benchmark of the overlap hot path.
+
+A step = one pass of the hot path over one synthetic batch: GEMM + tile signal +
+reordered store on the GEMM stream, per-group wait + consumer on the second
+stream, join, reorder+RMSNorm.  Workload: the large-square configuration the
+headline metric is quoted on (fp16, M=N=K=8192, 128x256 tiles, wave groups of
+256 tiles).  Prints one JSON line; `value` is GEMM flops / step time.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c2|c3|c4] [--dtype f16|bf16]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = 2516.6   # MI355X dense fp16/bf16 MFMA
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (M, N, K, BM, BN, dtype, group tiles, W, description)
+    "c5": (8192, 8192, 8192, 128, 256, "f16", 256, 0, "large square fp16 8192^3, 128x256 tiles, wave groups of 256 tiles"),
+    "c2": (4096, 4096, 512, 128, 128, "f16", 4, 0, "row-parallel K-slice fp16 4096x4096x512, 128x128 tiles, groups of 4 tiles"),
+    "c3": (8192, 8192, 3584, 256, 128, "bf16", 512, 0, "MLP down-projection bf16 8192x8192x3584, 256x128 tiles"),
+    "c4": (8192, 4096, 4096, 128, 128, "f16", 256, 8, "reduce-scatter layout fp16 8192x4096x4096, 8 row-chunk segments"),
+}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS))
+    ap.add_argument("--dtype", default=None, choices=["f16", "bf16"])
+    ap.add_argument("--swizzle", type=int, default=4)
+    ap.add_argument("--fused", type=int, default=0, help="1: one wait+reduce launch for all groups")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the collective is "
+              "replaced by a one-GPU consumer); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    os.environ.setdefault("FO_WAIT_MAX_POLLS", "200000000")  # a lost signal must not hang the GPU
+    import torch
+    import flashoverlap_amd as fo
+    from flashoverlap_amd import ops
+
+    torch.cuda.set_device(0)
+    M, N, K, BM, BN, dt, gtiles, W, desc = WORKLOADS[args.workload]
+    dt = args.dtype or dt
+    td = torch.float16 if dt == "f16" else torch.bfloat16
+    algo = fo._capi.find_algo(BM, BN, swizzle=args.swizzle)
+    TM, TN = M // BM, N // BN
+    T = TM * TN
+    cseg = fo.layout.cseg_from_waves(T, gtiles)
+    hint = fo._capi.schedule_order(algo, M, N)
+    RA = fo.layout.reorder_indices(T, hint, device="cuda").reshape(TM, TN)
+    RE = fo.layout.generate_row_mapping(M, N, BM, BN, cseg, W, device="cuda") if W else None
+
+    g = torch.Generator().manual_seed(0)
+    if args.workload == "c5":
+        A16 = ((torch.rand(M, K, generator=g) * 2 - 1) * K ** -0.5).to(td)
+        B16 = ((torch.rand(N, K, generator=g) * 2 - 1) * K ** -0.5).to(td)
+    else:
+        A16 = torch.randn(M, K, generator=g).to(td)
+        B16 = (torch.randn(N, K, generator=g) * K ** -0.5).to(td)
+    gamma16 = (1 + 0.01 * torch.randn(N, generator=g)).to(td)
+    A, B, gamma = A16.cuda(), B16.cuda(), gamma16.cuda()
+    Cp = torch.empty(M * N, device="cuda", dtype=td)
+    Cplain = torch.empty(M, N, device="cuda", dtype=td)
+    ACC = torch.zeros(M * N, device="cuda", dtype=td)
+    D = torch.empty(M // W, N, device="cuda", dtype=td) if W else None
+    bs = M // W if W else M
+    Y = torch.empty(bs, N, device="cuda", dtype=td)
+    MM = torch.zeros(fo.layout.counter_size(len(cseg), TM, TN), dtype=torch.int32, device="cuda")
+    cs_cpu = torch.tensor(cseg, dtype=torch.int32)
+    cs_gpu = cs_cpu.cuda()
+    eps = 1e-6
+
+    ov = ops.Overlap(rank=0, world=max(W, 1))
+    ov.set_accumulator(ACC)
+    ov.set_fused_consumer(bool(args.fused))
+
+    def norm():
+        if W:  # RMSNorm on segment 0 only
+            ops.reorder_rmsnorm(ACC.view(W, bs, N)[0], Y, gamma, BM // W, BN, 1, RA, eps=eps)
+        else:
+            ops.reorder_rmsnorm(Cp.view(M, N), Y, gamma, BM, BN, 1, RA, eps=eps)
+
+    def step_overlapped():
+        if W:
+            ov.gemm_reducescatter_overlap(A, B, Cp, D, MM, RA, RE, 1, cs_cpu, cs_gpu, algo)
+        else:
+            ov.gemm_allreduce_overlap(A, B, Cp, MM, RA, 1, cs_cpu, cs_gpu, algo)
+        norm()
+
+    def step_serial():  # signal-free GEMM, whole-C consumer, plain RMSNorm, one stream
+        ops.gemm(A, B, Cplain, algo)
+        if W:
+            ops.consumer_reduce_rs(Cplain.view(-1), ACC, W, (M // W) * N)
+            ops.rmsnorm(ACC.view(W, bs, N)[0], Y, gamma, eps=eps)
+        else:
+            ops.consumer_reduce(Cplain.view(-1), ACC)
+            ops.rmsnorm(Cplain, Y, gamma, eps=eps)
+
+    def gemm_alone():
+        ops.gemm(A, B, Cplain, algo)
+
+    def gemm_signal_alone():  # counters are not consumed here; cleared afterwards
+        ops.gemm_signal(A, B, Cp, MM, RA, cs_gpu, algo, RE=RE)
+
+    def consumer_alone():
+        ops.consumer_reduce(Cp, ACC)
+
+    def timed(fn, steps, warmup):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) * 1e3 / steps
+        return e0.elapsed_time(e1) / steps, wall
+
+    K_, W_ = args.steps, args.warmup
+    ms_step, wall_step = timed(step_overlapped, K_, W_)
+    ms_serial, _ = timed(step_serial, K_, W_)
+    ms_gemm, _ = timed(gemm_alone, K_, W_)
+    ms_signal, _ = timed(gemm_signal_alone, K_, W_)
+    MM.zero_()
+    ms_consumer, _ = timed(consumer_alone, K_, W_)
+    ms_norm, _ = timed(norm, K_, W_)
+    ACC.zero_()
+    torch.cuda.synchronize()
+
+    flops = 2.0 * M * N * K
+    achieved = flops / (ms_signal * 1e-3) / 1e12
+    out = {
+        "metric": "GEMM+signal+reorder TFLOP/s (% MFMA peak); overlapped vs serial time, 1 GPU",
+        "value": flops / (ms_step * 1e-3) / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": K_, "warmup": W_,
+        "ms_per_step": ms_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dt, "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {desc}", "M": M, "N": N, "K": K, "tile": [BM, BN],
+                   "groups": len(cseg), "algo": algo, "fused_consumer": bool(args.fused)},
+        "roofline": {"bound": "mfma", "kernel": "fo_gemm_kernel (signal epilogue)",
+                     "achieved": achieved, "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_TFLOPS, "traffic": None},
+        "times_ms": {"overlapped_step": ms_step, "overlapped_step_wall": wall_step,
+                     "serial_step": ms_serial, "gemm_alone": ms_gemm, "gemm_signal_alone": ms_signal,
+                     "consumer_alone": ms_consumer, "reorder_rmsnorm_alone": ms_norm},
+        "overlapped_vs_gemm_alone": ms_step / ms_gemm,
+        "overlapped_vs_serial": ms_step / ms_serial,
+        "consumer_GBps": 6.0 * M * N / (ms_consumer * 1e-3) / 1e9,
+        "reorder_rmsnorm_GBps": (4.0 * bs * N + 2.0 * N) / (ms_norm * 1e-3) / 1e9,
+        "hbm_peak_GBps": PEAK_HBM_GBS,
+    }
+
+    if not args.no_cpu_baseline:
+        from oracle import cpu_baseline
+        r = cpu_baseline.time_sample(A16, B16, gamma16, eps, target_seconds=15.0)
+        out["cpu_baseline"] = {"value": r["flops"] / r["seconds"] / 1e12, "unit": "TFLOP/s",
+                               "cores": r["threads"], "kind": "port",
+                               "sample": f"torch CPU fp32 matmul + RMSNorm on the first {r['rows']} of "
+                                         f"{M} rows of the same A (all of B), {r['seconds']:.1f} s; "
+                                         f"host has {os.cpu_count()} logical cpus"}
+    ov.close()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

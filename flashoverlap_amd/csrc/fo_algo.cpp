@@ -47,8 +47,14 @@ int fo_pick_raster(int algo, int M, int N, fo_raster *r) {
     const int bm = e->f[0], bn = e->f[1];
     if (M <= 0 || N <= 0) return FO_ERR_ARG;
     if (M % bm || N % bn) return FO_ERR_SHAPE;
+    // The workgroup (macro) tile may cover several reorder tiles: 256x256 when it
+    // divides the problem and leaves at least half a wave of workgroups.
     r->mtm = bm;
     r->mtn = bn;
+    if (M % 256 == 0 && N % 256 == 0 && (long)(M / 256) * (N / 256) >= 128) {
+        r->mtm = 256;
+        r->mtn = 256;
+    }
     r->grid_m = M / r->mtm;
     r->grid_n = N / r->mtn;
     r->panel = e->f[10] < r->grid_m ? e->f[10] : r->grid_m;

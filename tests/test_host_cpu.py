@@ -93,14 +93,21 @@ def test_schedule_order_is_a_permutation_with_local_waves(algo, M, N):
     bm, bn = _capi.algo_tile(algo)
     TM, TN = M // bm, N // bn
     assert sorted(order) == list(range(TM * TN))
-    if TM * TN >= 256 and (TM * TN) % 8 == 0:
+    # a workgroup covers `sub` reorder tiles when the 256x256 macro tile applies
+    macro = M % 256 == 0 and N % 256 == 0 and (M // 256) * (N // 256) >= 128
+    sub = (256 // bm) * (256 // bn) if macro else 1
+    wgs = [order[i:i + sub] for i in range(0, len(order), sub)]
+    if macro:
+        for w in wgs:   # the tiles of one workgroup form one 256x256 block
+            assert len({(t // TN) * bm // 256 for t in w}) == 1 and len({(t % TN) * bn // 256 for t in w}) == 1
+    if len(wgs) >= 256 and len(wgs) % 8 == 0:
         # one wave of 256 workgroups: 32 consecutive raster positions per XCD, so each
-        # XCD's share of the wave spans few distinct tile rows/columns
-        wave = order[:256]
+        # XCD's share of the wave spans few distinct macro-tile rows/columns
+        mt_m, mt_n = (256, 256) if macro else (bm, bn)
         for x in range(8):
-            mine = wave[x::8]
-            rows = {t // TN for t in mine}
-            cols = {t % TN for t in mine}
+            mine = [w[0] for w in wgs[:256][x::8]]
+            rows = {(t // TN) * bm // mt_m for t in mine}
+            cols = {(t % TN) * bn // mt_n for t in mine}
             assert len(rows) * len(cols) <= 64
 
 
