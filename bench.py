@@ -37,8 +37,18 @@ def main():
     ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS))
     ap.add_argument("--dtype", default=None, choices=["f16", "bf16"])
     ap.add_argument("--swizzle", type=int, default=4)
-    ap.add_argument("--fused", type=int, default=0, help="1: one wait+reduce launch for all groups")
+    ap.add_argument("--fused", type=int, default=-1,
+                    help="-1: library default (one wait+reduce launch above 16 groups), 0: two launches per "
+                         "group, 1: one launch")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--group-tiles", type=int, default=0, help="tiles per wave group (0: the workload's default)")
+    ap.add_argument("--no-group-sweep", action="store_true", help="skip the wave-group-size sweep (c5 only)")
+    ap.add_argument("--kernels-only", action="store_true",
+                    help="run each hot kernel alone on one stream and exit: for counter collection, which "
+                         "serialises dispatches and would stall a waiter that spins on another queue")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run a 256 MiB device-to-device copy five times (reference point for "
+                         "scaling the FETCH_SIZE / WRITE_SIZE counters) and exit")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the collective is "
@@ -51,7 +61,16 @@ def main():
     from flashoverlap_amd import ops
 
     torch.cuda.set_device(0)
+    if args.copy_calibration:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": src.numel(), "copy_bytes_written": dst.numel(), "copies": 5}))
+        return
     M, N, K, BM, BN, dt, gtiles, W, desc = WORKLOADS[args.workload]
+    gtiles = args.group_tiles or gtiles
     dt = args.dtype or dt
     td = torch.float16 if dt == "f16" else torch.bfloat16
     algo = fo._capi.find_algo(BM, BN, swizzle=args.swizzle)
@@ -84,7 +103,7 @@ def main():
 
     ov = ops.Overlap(rank=0, world=max(W, 1))
     ov.set_accumulator(ACC)
-    ov.set_fused_consumer(bool(args.fused))
+    ov.set_fused_consumer(args.fused)
 
     def norm():
         if W:  # RMSNorm on segment 0 only
@@ -132,6 +151,13 @@ def main():
         return e0.elapsed_time(e1) / steps, wall
 
     K_, W_ = args.steps, args.warmup
+    if args.kernels_only:
+        for fn in (gemm_alone, gemm_signal_alone, consumer_alone, norm):
+            timed(fn, K_, W_)
+            MM.zero_()
+        torch.cuda.synchronize()
+        print(json.dumps({"kernels_only": True, "steps": K_, "warmup": W_}))
+        return
     ms_step, wall_step = timed(step_overlapped, K_, W_)
     ms_serial, _ = timed(step_serial, K_, W_)
     ms_gemm, _ = timed(gemm_alone, K_, W_)
@@ -141,6 +167,27 @@ def main():
     ms_norm, _ = timed(norm, K_, W_)
     ACC.zero_()
     torch.cuda.synchronize()
+
+    # wave-group-size sweep (large square only): group sizes in waves of 256 tiles;
+    # 8 and 16 waves are a single group, i.e. the serial path (test/test.py:104)
+    sweep = []
+    if args.workload == "c5" and not args.no_group_sweep:
+        for waves in (1, 2, 4, 8, 16):
+            cs = fo.layout.cseg_from_waves(T, 256 * waves)
+            if len(cs) == 1:
+                sweep.append({"waves_per_group": waves, "groups": 1, "ms": ms_serial, "path": "serial"})
+                continue
+            c_cpu = torch.tensor(cs, dtype=torch.int32)
+            c_gpu = c_cpu.cuda()
+
+            def step_g():
+                ov.gemm_allreduce_overlap(A, B, Cp, MM, RA, 1, c_cpu, c_gpu, algo)
+                norm()
+            ms_g, _ = timed(step_g, K_, W_)
+            sweep.append({"waves_per_group": waves, "groups": len(cs), "ms": ms_g, "path": "overlapped",
+                          "vs_serial": ms_g / ms_serial, "vs_gemm_alone": ms_g / ms_gemm})
+        ACC.zero_()
+        torch.cuda.synchronize()
 
     flops = 2.0 * M * N * K
     achieved = flops / (ms_signal * 1e-3) / 1e12
@@ -153,7 +200,9 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dt, "data": "synthetic",
         "config": {"workload": f"{args.workload}: {desc}", "M": M, "N": N, "K": K, "tile": [BM, BN],
-                   "groups": len(cseg), "algo": algo, "fused_consumer": bool(args.fused)},
+                   "groups": len(cseg), "algo": algo,
+                   "consumer_launches": "per-group" if (args.fused == 0 or (args.fused < 0 and len(cseg) <= 16))
+                   else "one"},
         "roofline": {"bound": "mfma", "kernel": "fo_gemm_kernel (signal epilogue)",
                      "achieved": achieved, "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_TFLOPS, "traffic": None},
@@ -165,6 +214,7 @@ def main():
         "consumer_GBps": 6.0 * M * N / (ms_consumer * 1e-3) / 1e9,
         "reorder_rmsnorm_GBps": (4.0 * bs * N + 2.0 * N) / (ms_norm * 1e-3) / 1e9,
         "hbm_peak_GBps": PEAK_HBM_GBS,
+        "group_sweep": sweep,
     }
 
     if not args.no_cpu_baseline:

@@ -7,13 +7,14 @@
 namespace {
 
 // ------------------------------------------------------------------ wait
-// Replaces kernel_wait_flag (src/wait.cuh:5-9).  One lane polls with an
-// agent-scope acquire load and sleeps between polls; on equality a CAS resets
-// the counter to zero exactly as atomicCAS(addr, that, 0) does.
+// Replaces kernel_wait_flag (src/wait.cuh:5-9).  One lane polls with relaxed
+// agent-scope loads (an acquire per poll would invalidate the XCD's L2 under the
+// running GEMM every time) and sleeps between polls; on equality an acquiring
+// CAS resets the counter to zero exactly as atomicCAS(addr, that, 0) does.
 __global__ void fo_wait_kernel(int expect, int32_t *counter, long max_polls, int32_t *status) {
     long polls = 0;
     for (;;) {
-        int v = __hip_atomic_load(counter, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+        int v = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (v == expect) {
             int e = expect;
             if (__hip_atomic_compare_exchange_strong(counter, &e, 0, __ATOMIC_ACQ_REL,
@@ -42,38 +43,87 @@ __device__ __forceinline__ fo_u32x4 add8(fo_u32x4 a, fo_u32x4 b) {
     return fo_u32x4{o[0], o[1], o[2], o[3]};
 }
 
-// acc[q*seg_stride + i] += src[q*chunk + i] for q < W, i < chunk (16-byte units).
-template <typename Tag>
-__global__ __launch_bounds__(256) void fo_consumer_kernel(const fo_u32x4 *src, fo_u32x4 *acc, long chunk16,
-                                                          int W, long seg_stride16) {
-    const long total = chunk16 * W;
-    const long step = (long)gridDim.x * blockDim.x;
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += step) {
-        const long q = i / chunk16, o = i - q * chunk16;
-        fo_u32x4 *dst = acc + q * seg_stride16 + o;
-        *dst = add8<Tag>(*dst, src[i]);
+// The consumer runs beside the GEMM, whose workgroups each need most of a CU's
+// LDS and registers.  It therefore uses few, thin workgroups (256 lanes, no LDS,
+// a register budget that fits next to two GEMM wavefronts per SIMD) and gets
+// its bandwidth from depth instead: every lane keeps UNROLL 16-byte pieces of
+// both operands in flight.
+constexpr int CONSUMER_THREADS = 256;
+constexpr int CONSUMER_UNROLL = 8;
+constexpr int CONSUMER_MAX_BLOCKS = 256;  // a spinning grid of this size cannot occupy every CU three-deep
+// __launch_bounds__(256, 6) below caps the kernels at 80 VGPRs (six wavefronts per SIMD).
+
+// dst[i] += src[i] for i in [lo, hi) (16-byte units), the workgroup's lanes striding together.
+// RS: piece i belongs to chunk q = i / chunk16 and lands at dst + q*seg_stride16 + (i - q*chunk16).
+template <typename Tag, bool RS>
+__device__ __forceinline__ void reduce_range(const fo_u32x4 *src, fo_u32x4 *dst, long lo, long hi,
+                                             long chunk16, long seg_stride16, int tid, int nthreads) {
+    auto where = [&](long k) -> fo_u32x4 * {
+        if (!RS) return dst + k;
+        const long q = k / chunk16;
+        return dst + q * seg_stride16 + (k - q * chunk16);
+    };
+    constexpr int U = RS ? CONSUMER_UNROLL / 2 : CONSUMER_UNROLL;
+    long i = lo + tid;
+    const long step = (long)nthreads * U;
+    for (; i + (long)(U - 1) * nthreads < hi; i += step) {
+        fo_u32x4 a[U], b[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) a[u] = src[i + (long)u * nthreads];
+#pragma unroll
+        for (int u = 0; u < U; u++) b[u] = *where(i + (long)u * nthreads);
+#pragma unroll
+        for (int u = 0; u < U; u++) *where(i + (long)u * nthreads) = add8<Tag>(b[u], a[u]);
+    }
+    for (; i < hi; i += nthreads) {
+        fo_u32x4 *d = where(i);
+        *d = add8<Tag>(*d, src[i]);
     }
 }
 
-// One launch for all groups: every workgroup, for each group in order, has one
-// lane wait for MM[g] == cseg[g] (acquire), then all its lanes reduce their
-// slice of the group's contiguous range.  No workgroup waits for another one;
-// the last workgroup to leave resets every group counter (the CAS-to-zero of
-// src/wait.cuh:5-9, deferred to the end of the launch, before which nothing can
-// signal again) and clears workspace word 0.  Word 1 is set if a bounded poll
-// gave up.
+// acc[q*seg_stride + i] += src[q*chunk + i] for q < W, i < chunk (16-byte units).
 template <typename Tag>
-__global__ __launch_bounds__(512) void fo_wait_reduce_kernel(const fo_u32x4 *C, fo_u32x4 *ACC, int32_t *MM,
-                                                             const int32_t *cseg, int G,
-                                                             long tile16, int W, long seg_stride16,
-                                                             int32_t *ws, long max_polls) {
+__global__ __launch_bounds__(CONSUMER_THREADS, 6) void fo_consumer_kernel(const fo_u32x4 *src, fo_u32x4 *acc,
+                                                                       long chunk16, int W,
+                                                                       long seg_stride16) {
+    const long total = chunk16 * W;
+    const long per = (total + gridDim.x - 1) / gridDim.x;
+    const long lo = per * blockIdx.x;
+    const long hi = lo + per < total ? lo + per : total;
+    if (lo >= hi) return;
+    if (W <= 1)
+        reduce_range<Tag, false>(src, acc, lo, hi, 0, 0, threadIdx.x, blockDim.x);
+    else
+        reduce_range<Tag, true>(src, acc, lo, hi, chunk16, seg_stride16, threadIdx.x, blockDim.x);
+}
+
+// One launch for all groups.  The work is cut into items (group g, slice s of
+// that group's contiguous range); workgroup b owns items b, b+nb, b+2nb, ...
+// in ascending order, so different workgroups wait on different groups at the
+// same time and many small groups are consumed in parallel.  For its item a
+// workgroup has one lane poll MM[g] == cseg[g] (relaxed agent-scope loads, s_sleep
+// between polls, one acquire fence on success) and then all lanes reduce the slice.  No workgroup waits for
+// another one; the last workgroup to leave resets every group counter (the
+// CAS-to-zero of src/wait.cuh:5-9, deferred to the end of the launch, before
+// which nothing can signal again) and clears workspace word 0.  Word 1 is set
+// if a bounded poll gave up.
+template <typename Tag>
+__global__ __launch_bounds__(CONSUMER_THREADS, 6) void fo_wait_reduce_kernel(
+    const fo_u32x4 *C, fo_u32x4 *ACC, int32_t *MM, const int32_t *cseg, int G, long tile16, int W,
+    long seg_stride16, int slices, int32_t *ws, long max_polls) {
+    __shared__ int first_tile_s, last;
     const int nb = gridDim.x;
-    long base16 = 0;
-    for (int g = 0; g < G; g++) {
+    const long items = (long)G * slices;
+    int scanned_g = -1, scanned_first = 0;  // incremental exclusive prefix sum of cseg (items ascend)
+    for (long item = blockIdx.x; item < items; item += nb) {
+        const int g = (int)(item / slices), sl = (int)(item - (long)g * slices);
         const int cnt = cseg[g];
         if (threadIdx.x == 0) {
+            for (int j = scanned_g < 0 ? 0 : scanned_g; j < g; j++) scanned_first += cseg[j];
+            scanned_g = g;
+            first_tile_s = scanned_first;
             long polls = 0;
-            while (__hip_atomic_load(MM + g, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) != cnt) {
+            while (__hip_atomic_load(MM + g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != cnt) {
                 if (max_polls > 0 && ++polls >= max_polls) {  // debugging bound: flag and go on
                     __hip_atomic_store(ws + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     break;
@@ -82,29 +132,21 @@ __global__ __launch_bounds__(512) void fo_wait_reduce_kernel(const fo_u32x4 *C, 
             }
         }
         __syncthreads();
-        // The polling lane's acquire invalidated stale lines; repeat it for the
-        // other wavefronts' vector loads.
+        // Polling is relaxed (an acquire per poll would invalidate the L2 under the
+        // running GEMM every time); one acquire per item orders the group's data.
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-        const long n16 = (long)cnt * tile16;
         if (ACC) {
-            const long step = (long)nb * blockDim.x;
-            if (W <= 1) {
-                for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += step) {
-                    fo_u32x4 *dst = ACC + base16 + i;
-                    *dst = add8<Tag>(*dst, C[base16 + i]);
-                }
-            } else {
-                const long chunk16 = n16 / W;
-                for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += step) {
-                    const long q = i / chunk16, o = i - q * chunk16;
-                    fo_u32x4 *dst = ACC + q * seg_stride16 + base16 / W + o;
-                    *dst = add8<Tag>(*dst, C[base16 + i]);
-                }
-            }
+            const long base16 = (long)first_tile_s * tile16;
+            const long n16 = (long)cnt * tile16;
+            const long lo = n16 * sl / slices, hi = n16 * (sl + 1) / slices;
+            if (W <= 1)
+                reduce_range<Tag, false>(C + base16, ACC + base16, lo, hi, 0, 0, threadIdx.x, blockDim.x);
+            else
+                reduce_range<Tag, true>(C + base16, ACC + base16 / W, lo, hi, n16 / W, seg_stride16,
+                                        threadIdx.x, blockDim.x);
         }
-        base16 += n16;
+        __syncthreads();  // first_tile_s is rewritten for the next item
     }
-    __shared__ int last;
     if (threadIdx.x == 0) {
         int left = __hip_atomic_fetch_add(ws, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
         last = (left == nb - 1);
@@ -223,9 +265,9 @@ long default_max_polls() {
 }
 
 int consumer_grid(long n16) {
-    long blocks = (n16 + 256 * 4 - 1) / (256 * 4);  // about four 16-byte pieces per lane
+    long blocks = (n16 + CONSUMER_THREADS * CONSUMER_UNROLL - 1) / (CONSUMER_THREADS * CONSUMER_UNROLL);
     if (blocks < 1) blocks = 1;
-    if (blocks > 2048) blocks = 2048;
+    if (blocks > 2 * CONSUMER_MAX_BLOCKS) blocks = 2 * CONSUMER_MAX_BLOCKS;  // it does not spin: two per CU are fine
     return (int)blocks;
 }
 
@@ -255,7 +297,7 @@ extern "C" int fo_consumer_reduce_rs(int dtype, const void *src, void *acc, int6
     if (nelem % W || (nelem / W) % 8 || (W > 1 && seg_stride % 8)) return FO_ERR_SHAPE;
     if (((uintptr_t)src | (uintptr_t)acc) & 15) return FO_ERR_SHAPE;
     const long chunk16 = nelem / W / 8;
-    dim3 grid(consumer_grid(chunk16 * W)), block(256);
+    dim3 grid(consumer_grid(chunk16 * W)), block(CONSUMER_THREADS);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == FO_F16)
         hipLaunchKernelGGL(fo_consumer_kernel<fo_f16_tag>, grid, block, 0, s, (const fo_u32x4 *)src,
@@ -281,18 +323,23 @@ extern "C" int fo_wait_reduce_groups(int dtype, const void *C, void *ACC, int32_
     if (!MM || !cseg_dev || !workspace || G <= 0 || tile_elems <= 0 || W <= 0) return FO_ERR_ARG;
     if (ACC && !C) return FO_ERR_ARG;
     if (tile_elems % (8 * W) || (W > 1 && seg_stride % 8)) return FO_ERR_SHAPE;
-    if (nblocks <= 0) nblocks = 32;
-    if (nblocks > 256) nblocks = 256;
-    dim3 grid(nblocks), block(512);
+    // The grid spins until the GEMM signals, so it must never be able to crowd the
+    // GEMM's workgroups out of every CU: at most one thin workgroup per CU.
+    if (nblocks <= 0 || nblocks > CONSUMER_MAX_BLOCKS) nblocks = CONSUMER_MAX_BLOCKS;
+    // Slices per group: enough items to keep every workgroup busy on a large
+    // group, but no slice below one tile's worth of 16-byte pieces.
+    int slices = (nblocks + G - 1) / G;
+    if (slices < 1) slices = 1;
+    dim3 grid(nblocks), block(CONSUMER_THREADS);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == FO_F16)
         hipLaunchKernelGGL(fo_wait_reduce_kernel<fo_f16_tag>, grid, block, 0, s, (const fo_u32x4 *)C,
                            (fo_u32x4 *)ACC, MM, cseg_dev, G, (long)(tile_elems / 8), W,
-                           (long)(seg_stride / 8), workspace, default_max_polls());
+                           (long)(seg_stride / 8), slices, workspace, default_max_polls());
     else if (dtype == FO_BF16)
         hipLaunchKernelGGL(fo_wait_reduce_kernel<fo_bf16_tag>, grid, block, 0, s, (const fo_u32x4 *)C,
                            (fo_u32x4 *)ACC, MM, cseg_dev, G, (long)(tile_elems / 8), W,
-                           (long)(seg_stride / 8), workspace, default_max_polls());
+                           (long)(seg_stride / 8), slices, workspace, default_max_polls());
     else
         return FO_ERR_DTYPE;
     FO_LAUNCH_CHECK();

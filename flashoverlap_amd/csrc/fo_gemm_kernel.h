@@ -74,6 +74,18 @@ __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
+// 16-byte store that writes through the XCD's L2 to memory (system-scope cache
+// policy).  Used for the signalled epilogues: the tile must be visible to other
+// XCDs before its counter is bumped, and a tile that never becomes dirty in L2
+// makes the releasing write-back that precedes the signal nearly free.  The
+// compiler does not count this store in vmcnt; the epilogue waits explicitly.
+// The trailing s_nop covers the wait states gfx9 requires between a VMEM store
+// of more than 8 bytes and a VALU write of its data registers (the compiler
+// inserts them for its own stores but cannot see into inline assembly).
+__device__ __forceinline__ void store16_write_through(void *ptr, fo_u32x4 v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" : : "v"(ptr), "v"(v) : "memory");
+}
+
 #define FO_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 #define FO_GLB_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
 
@@ -408,7 +420,10 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
                 if (MODE == MODE_SCATTER) prow = p.RE[prow];
                 off = (size_t)prow * ldp + (size_t)(r % p.rLDN) * p.BN + n % p.BN;
             }
-            *reinterpret_cast<fo_u32x4 *>(p.C + off) = v;
+            if (MODE == MODE_PLAIN)
+                *reinterpret_cast<fo_u32x4 *>(p.C + off) = v;
+            else
+                store16_write_through(p.C + off, v);
         }
         __builtin_amdgcn_s_waitcnt(0xC07F);  // strip reads done before the next strip overwrites it
         __builtin_amdgcn_wave_barrier();

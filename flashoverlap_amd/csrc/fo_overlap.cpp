@@ -15,10 +15,20 @@ struct fo_overlap {
     int rank = 0, world = 1;
     void *acc = nullptr;
     int64_t acc_nelem = 0;
-    int fused = 0;
+    int fused = -1;  // -1: choose per call (one launch when there are many groups)
 };
 
 namespace {
+
+// Two launches per group cost a few microseconds each; beyond this many groups
+// the single wait+reduce launch is the faster consumer.
+constexpr int kFusedFromGroups = 16;
+
+int fused_grid(const fo_overlap *h, int G) {  // 0: per-group launches, otherwise workgroups of the one launch
+    if (h->fused < 0) return G > kFusedFromGroups ? 256 : 0;
+    if (h->fused == 1) return 256;
+    return h->fused;
+}
 
 int check_segments(const int32_t *cseg_host, int G, long tiles) {
     if (!cseg_host || G <= 0) return FO_ERR_SEGMENTS;
@@ -93,7 +103,7 @@ extern "C" int fo_overlap_set_accumulator(fo_overlap_t *h, void *acc, int64_t ne
 
 extern "C" int fo_overlap_set_fused_consumer(fo_overlap_t *h, int fused) {
     if (!h) return FO_ERR_ARG;
-    h->fused = fused ? 1 : 0;
+    h->fused = fused < 0 ? -1 : fused;
     return FO_OK;
 }
 
@@ -129,9 +139,10 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
                         h->gemm_stream);
     if (rc) return rc;  // nothing has been enqueued on the consumer stream yet
 
-    if (h->fused) {
+    const int fused = fused_grid(h, G);
+    if (fused) {
         rc = fo_wait_reduce_groups(dtype, C, h->acc, MM, cseg_dev, G, tile_elems, 1, 0, h->workspace,
-                                   0, h->comm_stream);
+                                   fused, h->comm_stream);
         if (rc) return rc;
     } else {
         int64_t off = 0;
@@ -178,15 +189,16 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
     uint16_t *c = static_cast<uint16_t *>(C);
     uint16_t *d = static_cast<uint16_t *>(D);
     uint16_t *acc = static_cast<uint16_t *>(h->acc);
-    if (h->fused) {
+    const int fused = fused_grid(h, G);
+    if (fused) {
         rc = fo_wait_reduce_groups(dtype, C, h->acc, MM, cseg_dev, G, tile_elems, W, seg_stride,
-                                   h->workspace, 0, h->comm_stream);
+                                   h->workspace, fused, h->comm_stream);
         if (rc) return rc;
     }
     int64_t off = 0;
     for (int i = 0; i < G; i++) {
         const int64_t n = cseg_host[i] * tile_elems;
-        if (!h->fused) {
+        if (!fused) {
             rc = fo_wait(cseg_host[i], MM + i, h->comm_stream);
             if (rc) return rc;
             if (acc) {

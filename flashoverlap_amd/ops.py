@@ -153,7 +153,7 @@ class Overlap:
                   "fo_overlap_set_accumulator")
 
     def set_fused_consumer(self, fused):
-        check(lib().fo_overlap_set_fused_consumer(self._h, int(bool(fused))),
+        check(lib().fo_overlap_set_fused_consumer(self._h, int(fused)),
               "fo_overlap_set_fused_consumer")
 
     def gemm(self, A, B, C, algo):

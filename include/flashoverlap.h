@@ -161,7 +161,10 @@ int fo_overlap_set_world(fo_overlap_t *h, int rank, int world);
  * reduces across ranks in place).  acc == NULL detaches it.  For W > 1 it is
  * [W, M/W, N] (seg_stride = M/W*N elements). */
 int fo_overlap_set_accumulator(fo_overlap_t *h, void *acc, int64_t nelem);
-/* fused != 0: use fo_wait_reduce_groups (one launch) instead of 2*G launches. */
+/* fused < 0 (default): chosen per call, one launch when there are more than 16
+ * groups; 0: always 2*G launches as the reference's host loop; 1: always one
+ * fo_wait_reduce_groups launch with the default grid; n > 1: the same with n
+ * workgroups. */
 int fo_overlap_set_fused_consumer(fo_overlap_t *h, int fused);
 fo_stream_t fo_overlap_comm_stream(fo_overlap_t *h);
 
