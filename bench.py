@@ -19,6 +19,9 @@ sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = 2516.6   # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch of the signal GEMM, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
+# profiles/gemm_c5_hbm_traffic.md (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 256 MiB copy).
+MEASURED_TRAFFIC_BYTES = {("c5", "f16"): 789059.4 * 1024 * 2.0 + 131136.0 * 1024}
 
 WORKLOADS = {
     # name: (M, N, K, BM, BN, dtype, group tiles, W, description)
@@ -205,7 +208,8 @@ def main():
                    else "one"},
         "roofline": {"bound": "mfma", "kernel": "fo_gemm_kernel (signal epilogue)",
                      "achieved": achieved, "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_TFLOPS, "traffic": None},
+                     "frac": achieved / PEAK_TFLOPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, dt))},
         "times_ms": {"overlapped_step": ms_step, "overlapped_step_wall": wall_step,
                      "serial_step": ms_serial, "gemm_alone": ms_gemm, "gemm_signal_alone": ms_signal,
                      "consumer_alone": ms_consumer, "reorder_rmsnorm_alone": ms_norm},
