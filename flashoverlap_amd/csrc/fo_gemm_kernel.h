@@ -86,6 +86,25 @@ __device__ __forceinline__ void store16_write_through(void *ptr, fo_u32x4 v) {
     asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" : : "v"(ptr), "v"(v) : "memory");
 }
 
+// One direct-to-LDS load of 16 bytes per lane in the saddr form: global address =
+// wave-uniform base (SGPR pair) + 32-bit per-lane byte offset; LDS address =
+// M0 + lane * 16.  Written as assembly because the compiler materialises a
+// 64-bit VGPR address for the intrinsic (two VALU instructions per load, which
+// steal issue slots from the MFMAs); it does not track these loads in vmcnt,
+// the main loop waits explicitly.  The s_nop covers the M0 write -> LDS-DMA
+// wait state.
+__device__ __forceinline__ void dma_load16(const __attribute__((address_space(1))) char *base, unsigned lane_off,
+                                           unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_addr), "v"(lane_off), "s"(base)
+                 : "memory");
+}
+
+// cache policy bits of the operand loads (gfx940 encoding: 1 = sc0, 2 = nt, 16 = sc1)
+#ifndef FO_LOAD_CPOL
+#define FO_LOAD_CPOL 0
+#endif
 #define FO_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 #define FO_GLB_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
 
@@ -107,6 +126,7 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
     static_assert(STAGES >= 2, "ring depth");
 
     extern __shared__ fo_u32x4 smem[];
+    const unsigned smem_lds = (unsigned)(uintptr_t)FO_LDS_PTR(smem);  // LDS byte address of the ring
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -161,25 +181,26 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
     // of its first block holds for all of them.
     const int lrow = lane / CH;
     const int lchunk = (lane % CH) ^ (((wave * (64 / CH) + lrow) >> SWZ_SHIFT) & (CH - 1));
-    const fo_u32x4 *Ag = reinterpret_cast<const fo_u32x4 *>(p.A) +
-                         ((size_t)pm * MTM + wave * (64 / CH) + lrow) * lda16 + lchunk;
-    const fo_u32x4 *Bg = reinterpret_cast<const fo_u32x4 *>(p.B) +
-                         ((size_t)pn * MTN + wave * (64 / CH) + lrow) * ldb16 + lchunk;
-    const size_t a_blk_stride = (size_t)NW * (64 / CH) * lda16;  // rows between a wave's consecutive blocks
-    const size_t b_blk_stride = (size_t)NW * (64 / CH) * ldb16;
+    // Global addresses = wave-uniform base (SGPRs, advanced with scalar adds) + one
+    // loop-invariant 32-bit per-lane byte offset, so the loads use the saddr form
+    // and the K loop carries no vector address arithmetic.
+    typedef const __attribute__((address_space(1))) char *gptr_t;
+    gptr_t Ab = (gptr_t)(p.A) + ((size_t)pm * MTM + wave * (64 / CH)) * p.lda * 2;
+    gptr_t Bb = (gptr_t)(p.B) + ((size_t)pn * MTN + wave * (64 / CH)) * p.ldb * 2;
+    const unsigned a_lane = (unsigned)(lrow * p.lda * 2 + lchunk * 16);
+    const unsigned b_lane = (unsigned)(lrow * p.ldb * 2 + lchunk * 16);
+    const size_t a_blk_bytes = (size_t)NW * (64 / CH) * p.lda * 2;  // between a wave's consecutive blocks
+    const size_t b_blk_bytes = (size_t)NW * (64 / CH) * p.ldb * 2;
 
     // Issue the loads of K step kt into ring slot s (PA + PB instructions per wavefront).
     auto issue = [&](int kt, int s) {
-        fo_u32x4 *as = smem + s * STAGE16 + wave * 64;
-        fo_u32x4 *bs = as + MTM * CH;
+        const unsigned as = smem_lds + (unsigned)(s * STAGE16 + wave * 64) * 16;  // LDS byte addresses
+        const unsigned bs = as + MTM * CH * 16;
+        gptr_t ak = Ab + (size_t)kt * (BK * 2), bk = Bb + (size_t)kt * (BK * 2);
 #pragma unroll
-        for (int i = 0; i < PA; i++)
-            __builtin_amdgcn_global_load_lds(FO_GLB_PTR(Ag + i * a_blk_stride + kt * CH),
-                                             FO_LDS_PTR(as + i * NW * 64), 16, 0, 0);
+        for (int i = 0; i < PA; i++) dma_load16(ak + i * a_blk_bytes, a_lane, as + i * NW * 1024);
 #pragma unroll
-        for (int i = 0; i < PB; i++)
-            __builtin_amdgcn_global_load_lds(FO_GLB_PTR(Bg + i * b_blk_stride + kt * CH),
-                                             FO_LDS_PTR(bs + i * NW * 64), 16, 0, 0);
+        for (int i = 0; i < PB; i++) dma_load16(bk + i * b_blk_bytes, b_lane, bs + i * NW * 1024);
     };
 
     constexpr int P = PA + PB;   // load instructions per wavefront and stage
@@ -232,8 +253,13 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
     // per k-step, pinned MFMA-first with the memory instructions in its shadow.
     // STEADY additionally means kt >= STAGES-1 and that a prefetch is still due,
     // so the number of younger loads in flight at the wait is a constant.
-    auto kstep = [&](auto steady, int kt, int slot, int nslot) {
+    // With two slots the loop is unrolled by two and the slot is a compile-time
+    // constant (slot_tag >= 0), which makes every LDS address loop-invariant.
+    auto kstep = [&](auto steady, auto slot_tag, int kt, int slot_rt, int nslot_rt) {
         constexpr bool STEADY = decltype(steady)::value;
+        constexpr int SLOT_C = decltype(slot_tag)::value;
+        const int slot = SLOT_C >= 0 ? SLOT_C : slot_rt;
+        const int nslot = SLOT_C >= 0 ? (SLOT_C ^ 1) : nslot_rt;
         const fo_u32x4 *st = smem + slot * STAGE16;
 #pragma unroll
         for (int kk = 0; kk < KK; kk++) {
@@ -276,21 +302,30 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
         }
     };
 
+    using dyn = std::integral_constant<int, -1>;
     int slot = 0;  // ring slot of K step kt
     int kt = 0;
     for (; kt < STAGES - 1 && kt < KT; kt++) {
         const int nslot = slot + 1 == STAGES ? 0 : slot + 1;
-        kstep(std::false_type{}, kt, slot, nslot);
+        kstep(std::false_type{}, dyn{}, kt, slot, nslot);
         slot = nslot;
     }
-    for (; kt + STAGES + PFD < KT; kt++) {
-        const int nslot = slot + 1 == STAGES ? 0 : slot + 1;
-        kstep(std::true_type{}, kt, slot, nslot);
-        slot = nslot;
+    if constexpr (STAGES == 2) {
+        // here kt == 1 (slot 1) when KT > 1
+        for (; kt + 1 + STAGES + PFD < KT; kt += 2) {
+            kstep(std::true_type{}, std::integral_constant<int, 1>{}, kt, 1, 0);
+            kstep(std::true_type{}, std::integral_constant<int, 0>{}, kt + 1, 0, 1);
+        }
+    } else {
+        for (; kt + STAGES + PFD < KT; kt++) {
+            const int nslot = slot + 1 == STAGES ? 0 : slot + 1;
+            kstep(std::true_type{}, dyn{}, kt, slot, nslot);
+            slot = nslot;
+        }
     }
     for (; kt < KT; kt++) {
         const int nslot = slot + 1 == STAGES ? 0 : slot + 1;
-        kstep(std::false_type{}, kt, slot, nslot);
+        kstep(std::false_type{}, dyn{}, kt, slot, nslot);
         slot = nslot;
     }
     }
@@ -370,6 +405,113 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
         for (; kt < KT; kt++) kstep(std::false_type{}, kt);
 #undef FO_GLOAD
 #undef FO_LSTORE
+    }
+
+    // ---- main loop, register-staged loader with two register sets (LOADER == 2):
+    // HBM -> VGPR -> LDS through ds_write_b128 (128 B/clk, twice the rate at which
+    // direct-to-LDS loads occupy the LDS), two LDS slots.  Stage s is requested
+    // in K step s-3 (k-steps 2,3), written to LDS in K step s-1 (k-steps 0,1)
+    // and consumed in K step s, so a load has about 1.5 K steps to arrive and
+    // the memory instructions are spread evenly between the MFMAs.
+    if constexpr (LOADER == 2 || LOADER == 3) {
+        constexpr int NSETS = LOADER == 2 ? 2 : 1;  // register sets: a load has NSETS - 0.5 K steps to arrive
+        static_assert(KK == 4, "the two-set loader is scheduled for BK = 64");
+        constexpr int NT = NW * 64;
+        constexpr int RP = NT / CH;  // tile rows covered by one pass of the whole workgroup
+        constexpr int LA = MTM / RP, LB = MTN / RP, NL = LA + LB;
+        static_assert(RP % 32 == 0 && MTM % RP == 0 && MTN % RP == 0 && NL % 2 == 0, "loader split");
+        const int lc = tid % CH, lr = tid / CH;
+        const int lsw = lc ^ ((lr >> SWZ_SHIFT) & (CH - 1));
+        // Addresses as a wave-uniform base (SGPRs, advanced with scalar adds) plus one
+        // 32-bit per-lane byte offset, so the loads use the saddr form and no VGPRs
+        // are spent on 64-bit pointers.
+        const char *Ab = reinterpret_cast<const char *>(p.A) + (size_t)pm * MTM * p.lda * 2;
+        const char *Bb = reinterpret_cast<const char *>(p.B) + (size_t)pn * MTN * p.ldb * 2;
+        const unsigned a_lane = (unsigned)(lr * p.lda * 2 + lc * 16);
+        const unsigned b_lane = (unsigned)(lr * p.ldb * 2 + lc * 16);
+        const size_t apass = (size_t)RP * p.lda * 2, bpass = (size_t)RP * p.ldb * 2;  // bytes
+        fo_u32x4 rs[NSETS][NL];
+        // loads / stores i in [lo_, hi_) of one stage; i < LA are A rows, the rest B rows
+#define FO_GLOAD2(set_, kt_, lo_, hi_)                                                          \
+    _Pragma("unroll") for (int i = (lo_); i < (hi_); i++)                                       \
+        rs[set_][i] = i < LA ? *reinterpret_cast<const fo_u32x4 *>(Ab + i * apass + (size_t)(kt_) * (BK * 2) + a_lane) \
+                             : *reinterpret_cast<const fo_u32x4 *>(Bb + (i - LA) * bpass + (size_t)(kt_) * (BK * 2) + b_lane);
+#define FO_LSTORE2(set_, slot_, lo_, hi_)                                                       \
+    _Pragma("unroll") for (int i = (lo_); i < (hi_); i++)                                       \
+        smem[(slot_) * STAGE16 + (i < LA ? (lr + i * RP) * CH : MTM * CH + (lr + (i - LA) * RP) * CH) + lsw] = \
+            rs[set_][i];
+
+        FO_GLOAD2(0, 0, 0, NL)
+        if (NSETS == 2 && KT > 1) {
+            FO_GLOAD2(NSETS - 1, 1, 0, NL)
+        }
+        FO_LSTORE2(0, 0, 0, NL)
+        if (KT > NSETS) {
+            FO_GLOAD2(0, NSETS, 0, NL)
+        }
+        __syncthreads();
+        FO_LOAD_FRAGS(0, smem, 0)
+
+        // K step kt with parity PAR = kt & 1; the set that holds stage kt+1 is PAR ^ 1.
+        auto kstep = [&](auto steady, auto parity, int kt) {
+            constexpr bool STEADY = decltype(steady)::value;  // kt + 3 < KT
+            constexpr int PAR = decltype(parity)::value;
+            constexpr int NXT = PAR ^ 1;               // LDS slot of stage kt+1
+            constexpr int SET = NSETS == 2 ? NXT : 0;  // register set of stage kt+1, refilled with stage kt+1+NSETS
+            const fo_u32x4 *st = smem + PAR * STAGE16;
+#pragma unroll
+            for (int kk = 0; kk < KK; kk++) {
+                if (kk + 1 < KK) {
+                    FO_LOAD_FRAGS((kk + 1) & 1, st, kk + 1)
+                }
+                if (kk < 2 && (STEADY || kt + 1 < KT)) {
+                    FO_LSTORE2(SET, NXT, kk * (NL / 2), (kk + 1) * (NL / 2))
+                }
+                if (kk == 2 && (STEADY || kt + 1 + NSETS < KT)) {
+                    FO_GLOAD2(SET, kt + 1 + NSETS, 0, NL / 2)
+                }
+                if (kk == 3 && (STEADY || kt + 1 < KT)) {
+                    // own reads of this slot and own writes of the other one are
+                    // complete; the barrier makes that true for the workgroup
+                    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+                    __builtin_amdgcn_s_barrier();
+                    asm volatile("" ::: "memory");
+                    FO_LOAD_FRAGS((kk + 1) & 1, smem + NXT * STAGE16, 0)
+                }
+                if (kk == 3 && (STEADY || kt + 1 + NSETS < KT)) {
+                    FO_GLOAD2(SET, kt + 1 + NSETS, NL / 2, NL)
+                }
+                FO_MFMAS(kk)
+                if (STEADY && !(DBG & 16)) {
+                    constexpr int NO = NL / 2;  // ds_writes (k-steps 0,1) or global loads (2,3) in this region
+                    static_assert(NR <= NM && NO <= NM, "at most one read and one write/load per MFMA");
+#pragma unroll
+                    for (int t = 0; t < NM; t++) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        if (((t + 1) * NR) / NM > (t * NR) / NM) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                        if (((t + 1) * NO) / NM > (t * NO) / NM) {
+                            if (kk < 2)
+                                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                            else
+                                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                        }
+                    }
+                }
+            }
+        };
+        int kt = 0;
+        for (; kt + 4 < KT; kt += 2) {
+            kstep(std::true_type{}, std::integral_constant<int, 0>{}, kt);
+            kstep(std::true_type{}, std::integral_constant<int, 1>{}, kt + 1);
+        }
+        for (; kt < KT; kt++) {
+            if (kt & 1)
+                kstep(std::false_type{}, std::integral_constant<int, 1>{}, kt);
+            else
+                kstep(std::false_type{}, std::integral_constant<int, 0>{}, kt);
+        }
+#undef FO_GLOAD2
+#undef FO_LSTORE2
     }
 
 #undef FO_LOAD_FRAGS
