@@ -227,7 +227,7 @@ def main():
         out["cpu_baseline"] = {"value": r["flops"] / r["seconds"] / 1e12, "unit": "TFLOP/s",
                                "cores": r["threads"], "kind": "port",
                                "sample": f"torch CPU fp32 matmul + RMSNorm on the first {r['rows']} of "
-                                         f"{M} rows of the same A (all of B), {r['seconds']:.1f} s; "
+                                         f"{M} rows of the same A (all of B), {r['passes']} passes, {r['seconds']:.1f} s; "
                                          f"host has {os.cpu_count()} logical cpus"}
     ov.close()
     print(json.dumps(out))

@@ -20,6 +20,7 @@ SIGNATURES = {
     "fo_algo_count": (c_int, []),
     "fo_algo_info": (c_int, [c_int, vp]),
     "fo_schedule_order": (c_int, [c_int, c_int, c_int, vp]),
+    "fo_workgroup_tiles": (c_int, [c_int, c_int, c_int, vp, vp]),
     "fo_gemm": (c_int, [c_int, c_int, c_int, c_int, vp, vp, vp, c_int, vp]),
     "fo_gemm_signal": (c_int, [c_int, c_int, c_int, c_int, c_int, vp, c_int, vp, vp, vp, vp, vp,
                                c_int, c_int, vp]),
@@ -116,3 +117,11 @@ def schedule_order(algo, M, N):
     buf = (ctypes.c_int32 * T)()
     check(lib().fo_schedule_order(int(algo), M, N, buf), "fo_schedule_order")
     return list(buf)
+
+
+def wave_tiles(algo, M, N, cus=256):
+    """Reorder tiles one wave of the chip completes: CUs x tiles per workgroup."""
+    per = ctypes.c_int32()
+    wgs = ctypes.c_int32()
+    check(lib().fo_workgroup_tiles(int(algo), M, N, ctypes.byref(per), ctypes.byref(wgs)), "fo_workgroup_tiles")
+    return cus * per.value

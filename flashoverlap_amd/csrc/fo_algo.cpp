@@ -94,6 +94,16 @@ extern "C" int fo_schedule_order(int algo, int M, int N, int32_t *order) {
     return FO_OK;
 }
 
+extern "C" int fo_workgroup_tiles(int algo, int M, int N, int32_t *tiles_per_workgroup, int32_t *workgroups) {
+    fo_raster r;
+    int rc = fo_pick_raster(algo, M, N, &r);
+    if (rc) return rc;
+    const fo_algo_entry *e = fo_algo_lookup(algo);
+    if (tiles_per_workgroup) *tiles_per_workgroup = (r.mtm / e->f[0]) * (r.mtn / e->f[1]);
+    if (workgroups) *workgroups = r.grid_m * r.grid_n;
+    return FO_OK;
+}
+
 extern "C" int fo_version(void) { return 100; }
 
 extern "C" const char *fo_error_string(int code) {

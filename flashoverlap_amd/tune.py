@@ -218,3 +218,66 @@ def exhaustive_search(M, N, K, algo, wave, hint, dtype=torch.float16, reps=50):
         if ms < best_ms:
             best, best_ms = cseg, ms
     return best, best_ms, table
+
+
+# ------------------------------------------------------------------ command line
+def tune_shape(M, N, K, comm_op="all_reduce", predictive=False, dtype=torch.float16, directory=None,
+               candidates=None, reps=100, quiet=False):
+    """The reference's three tuning steps for one shape on one GPU, writing the same
+    JSON files: GEMM candidates (tune/gen_config.py), consumer bandwidth curve
+    (tune/bandwidth.py), wave-group search (tune/search.py).  Returns the solution dict."""
+    import os
+    from . import config
+    say = (lambda *a: None) if quiet else print
+    BMs, BNs, durs, algos = profile_gemm_configs(M, N, K, dtype, top=candidates or 10, warmup=10, reps=reps)
+    path = config.save_gemm_candidates(M, N, K, BMs, BNs, durs, algos, directory=directory)
+    say("GEMM candidates ->", path)
+    # forced for large outputs, as tune/search.py:519
+    predictive = predictive or M * N > 33554432
+    curve = None
+    if predictive:
+        curve = consumer_bandwidth_curve(dtype)
+        cdir = directory or config.DEFAULT_DIR
+        os.makedirs(cdir, exist_ok=True)
+        torch.save(curve, os.path.join(cdir, f"bandwidth_{comm_op}_tp1.pt"))
+    BM, BN, dur, algo = BMs[0], BNs[0], durs[0], algos[0]
+    tile_num = (M // BM) * (N // BN)
+    wave = _capi.wave_tiles(algo, M, N)
+    analytic = _capi.schedule_order(algo, M, N)
+    hint = analytic
+    if div_up(tile_num, wave) <= N // BN - 1:   # monitor mode keeps its order counter at MM[TN-1]
+        ok, measured = measured_hint(M, N, K, algo, wave, dtype)
+        say("monitor-mode hint consistent with the wave structure:", ok)
+        if ok:
+            hint = measured
+    if predictive:
+        cseg, est = predictive_search(M, N, dur, curve.numpy(), tile_num, wave)
+        say("predicted latency %.4f ms for cSeg %s" % (est, cseg))
+    else:
+        cseg, ms, table = exhaustive_search(M, N, K, algo, wave, hint, dtype, reps=max(10, reps // 4))
+        for c, t in table:
+            say(c, "%.4f" % t)
+    ms = time_overlap(M, N, K, algo, cseg, hint, dtype, warmup=10, reps=reps)
+    say("searched latency %.4f ms, best cSeg %s" % (ms, cseg))
+    path = config.save_solution(M, N, K, BM, BN, dur, algo, hint, cseg, directory=directory)
+    say("solution ->", path)
+    return config.load_solution(M, N, K, directory=directory)
+
+
+def main(argv=None):
+    import argparse
+    ap = argparse.ArgumentParser(description="wave-group tuning on one GPU (tune/search.py:506-525)")
+    ap.add_argument("--m", type=int, default=4096)
+    ap.add_argument("--k", type=int, default=8192)
+    ap.add_argument("--n", type=int, default=8192)
+    ap.add_argument("--comm_op", type=str, default="all_reduce")
+    ap.add_argument("--predictive_search", type=bool, default=False)  # any non-empty string is true, as in the reference
+    ap.add_argument("--dtype", default="f16", choices=["f16", "bf16"])
+    ap.add_argument("--path", default=None, help="directory of the config JSONs")
+    a = ap.parse_args(argv)
+    tune_shape(a.m, a.n, a.k, a.comm_op, a.predictive_search,
+               torch.float16 if a.dtype == "f16" else torch.bfloat16, a.path)
+
+
+if __name__ == "__main__":
+    main()

@@ -55,6 +55,12 @@ int fo_algo_info(int algo, int32_t info[12]);
  * mode; order must hold (M/BM)*(N/BN) ints (host memory). */
 int fo_schedule_order(int algo, int M, int N, int32_t *order);
 
+/* How the GEMM kernels cover the problem: reorder tiles per workgroup (the
+ * workgroup tile may span several BM x BN tiles) and the number of workgroups.
+ * One wave of the 256-CU chip completes 256 * tiles_per_workgroup tiles; the
+ * reference's tuner uses sm_count - 2 tiles per wave (tune/search.py:404). */
+int fo_workgroup_tiles(int algo, int M, int N, int32_t *tiles_per_workgroup, int32_t *workgroups);
+
 /* ---- GEMM -------------------------------------------------------------
  * C[M,N] = A[M,K] . B[N,K]^T, 16-bit in/out, fp32 accumulate.
  * Replaces gemm_func_table[Algo](M,N,K,A,B,C,stream), src/gemm/gemm.cu:23-110,

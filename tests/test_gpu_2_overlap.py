@@ -303,3 +303,44 @@ def test_config4_reduce_scatter_layout(fo):
 @pytest.mark.parametrize("dtype", [F16, BF16])
 def test_config5_large_square(fo, dtype):
     _full_size_case(fo, dtype, 128, 256, 8192, 8192, 8192, [256] * 8, swizzle=4, dist="uniform")
+
+
+# ---------------------------------------------------------------- tuning pipeline
+def test_tuning_pipeline_writes_a_usable_config(fo, tmp_path):
+    """Stage-1 candidates, monitor-mode hint, exhaustive search over the wave
+    compositions, stage-2 JSON; the tuned config then drives a correct overlapped run."""
+    from flashoverlap_amd import tune, config
+    M, N, K = 8192, 4096, 128
+    sol = tune.tune_shape(M, N, K, directory=str(tmp_path), candidates=3, reps=8, quiet=True)
+    assert set(sol) >= {"hint", "cSeg", "rLDN", "BM", "BN", "dur", "Algo"} and sol["rLDN"] == 1
+    BM, BN, algo = sol["BM"], sol["BN"], sol["Algo"]
+    T = (M // BM) * (N // BN)
+    assert sum(sol["cSeg"]) == T and sorted(sol["hint"]) == list(range(T))
+    assert fo._capi.algo_tile(algo) == (BM, BN)
+    TM, TN = M // BM, N // BN
+    RA = fo.layout.reorder_indices(T, sol["hint"], device="cuda").reshape(TM, TN)
+    A, _ = seeded((M, K), F16, 90)
+    B, _ = seeded((N, K), F16, 91, scale=K ** -0.5)
+    plain = torch.empty(M, N, device="cuda", dtype=torch.float16)
+    Cp = torch.empty(M * N, device="cuda", dtype=torch.float16)
+    MM = torch.zeros(fo.layout.counter_size(len(sol["cSeg"]), TM, TN), dtype=torch.int32, device="cuda")
+    cs = torch.tensor(sol["cSeg"], dtype=torch.int32)
+    ov = fo.ops.Overlap()
+    ov.gemm(A, B, plain, algo)
+    ov.gemm_allreduce_overlap(A, B, Cp, MM, RA, 1, cs, cs.cuda(), algo)
+    torch.cuda.synchronize()
+    assert torch.equal(fo.layout.unpermute(Cp, M, N, BM, BN, RA), plain) and (MM == 0).all()
+    ov.close()
+
+
+def test_predictive_search_on_measured_curve(fo):
+    from flashoverlap_amd import tune
+    curve = tune.consumer_bandwidth_curve(points=12, warmup=2, reps=5).numpy()
+    assert curve.shape == (12, 2) and (curve[:, 1] > 0).all()
+    assert curve[-1, 1] > curve[0, 1] * 0.5          # GiB/ms; large sizes are not slower than tiny ones
+    M = N = 8192
+    algo = fo._capi.find_algo(256, 128, swizzle=4)
+    wave = fo._capi.wave_tiles(algo, M, N)
+    assert wave == 512                                # 256 CUs x two 256x128 tiles per 256x256 workgroup
+    cseg, est = tune.predictive_search(M, N, 0.4, curve, 2048, wave)
+    assert sum(cseg) == 2048 and est > 0.4
