@@ -49,13 +49,28 @@ __device__ __forceinline__ fo_u32x4 add8(fo_u32x4 a, fo_u32x4 b) {
 // its bandwidth from depth instead: every lane keeps UNROLL 16-byte pieces of
 // both operands in flight.
 constexpr int CONSUMER_THREADS = 256;
-constexpr int CONSUMER_UNROLL = 8;
+constexpr int CONSUMER_UNROLL = 4;
 constexpr int CONSUMER_MAX_BLOCKS = 256;  // a spinning grid of this size cannot occupy every CU three-deep
-// __launch_bounds__(256, 6) below caps the kernels at 80 VGPRs (six wavefronts per SIMD).
+// __launch_bounds__(256, 8) below caps the kernels at 64 VGPRs: the signalling GEMM holds two
+// wavefronts of up to 224 registers on each SIMD, which leaves 64 of the 512 for one consumer wavefront.
+
+// 16-byte load that bypasses the non-coherent caches (system-scope cache
+// policy).  The fused consumer reads tiles that workgroups on other XCDs wrote
+// through to memory moments ago; reading them this way needs no acquire fence,
+// whose L2 invalidation would throw the running GEMM's operand panels out of
+// this XCD's L2.  `base` is wave-uniform, `off` a per-lane byte offset.
+__device__ __forceinline__ fo_u32x4 load16_coherent(const fo_u32x4 *base, unsigned off) {
+    __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, 0x7fffffff, 0x00027000);
+    return __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, /*sc0 | sc1*/ 17);
+}
 
 // dst[i] += src[i] for i in [lo, hi) (16-byte units), the workgroup's lanes striding together.
 // RS: piece i belongs to chunk q = i / chunk16 and lands at dst + q*seg_stride16 + (i - q*chunk16).
-template <typename Tag, bool RS>
+// COHERENT: src is read past the caches (see load16_coherent).  Everything else is
+// streamed with the non-temporal cache policy: the data is touched once, and
+// lines kept for it would push the operand panels of a GEMM running beside the
+// consumer out of the L2.
+template <typename Tag, bool RS, bool COHERENT>
 __device__ __forceinline__ void reduce_range(const fo_u32x4 *src, fo_u32x4 *dst, long lo, long hi,
                                              long chunk16, long seg_stride16, int tid, int nthreads) {
     auto where = [&](long k) -> fo_u32x4 * {
@@ -63,27 +78,34 @@ __device__ __forceinline__ void reduce_range(const fo_u32x4 *src, fo_u32x4 *dst,
         const long q = k / chunk16;
         return dst + q * seg_stride16 + (k - q * chunk16);
     };
+    auto fetch = [&](long first, int u) -> fo_u32x4 {  // src[first + tid + u * nthreads], first wave-uniform
+        if (COHERENT) return load16_coherent(src + first, (unsigned)(tid + u * nthreads) * 16u);
+        return __builtin_nontemporal_load(src + first + tid + (long)u * nthreads);
+    };
     constexpr int U = RS ? CONSUMER_UNROLL / 2 : CONSUMER_UNROLL;
-    long i = lo + tid;
+    long first = lo;
     const long step = (long)nthreads * U;
-    for (; i + (long)(U - 1) * nthreads < hi; i += step) {
+    for (; first + step <= hi; first += step) {
+        const long i = first + tid;
         fo_u32x4 a[U], b[U];
 #pragma unroll
-        for (int u = 0; u < U; u++) a[u] = src[i + (long)u * nthreads];
+        for (int u = 0; u < U; u++) a[u] = fetch(first, u);
 #pragma unroll
-        for (int u = 0; u < U; u++) b[u] = *where(i + (long)u * nthreads);
+        for (int u = 0; u < U; u++) b[u] = __builtin_nontemporal_load(where(i + (long)u * nthreads));
 #pragma unroll
-        for (int u = 0; u < U; u++) *where(i + (long)u * nthreads) = add8<Tag>(b[u], a[u]);
+        for (int u = 0; u < U; u++) __builtin_nontemporal_store(add8<Tag>(b[u], a[u]), where(i + (long)u * nthreads));
     }
-    for (; i < hi; i += nthreads) {
-        fo_u32x4 *d = where(i);
-        *d = add8<Tag>(*d, src[i]);
+    for (; first < hi; first += nthreads) {
+        if (first + tid < hi) {
+            fo_u32x4 *d = where(first + tid);
+            __builtin_nontemporal_store(add8<Tag>(__builtin_nontemporal_load(d), fetch(first, 0)), d);
+        }
     }
 }
 
 // acc[q*seg_stride + i] += src[q*chunk + i] for q < W, i < chunk (16-byte units).
 template <typename Tag>
-__global__ __launch_bounds__(CONSUMER_THREADS, 6) void fo_consumer_kernel(const fo_u32x4 *src, fo_u32x4 *acc,
+__global__ __launch_bounds__(CONSUMER_THREADS, 8) void fo_consumer_kernel(const fo_u32x4 *src, fo_u32x4 *acc,
                                                                        long chunk16, int W,
                                                                        long seg_stride16) {
     const long total = chunk16 * W;
@@ -92,25 +114,38 @@ __global__ __launch_bounds__(CONSUMER_THREADS, 6) void fo_consumer_kernel(const 
     const long hi = lo + per < total ? lo + per : total;
     if (lo >= hi) return;
     if (W <= 1)
-        reduce_range<Tag, false>(src, acc, lo, hi, 0, 0, threadIdx.x, blockDim.x);
+        reduce_range<Tag, false, false>(src, acc, lo, hi, 0, 0, threadIdx.x, blockDim.x);
     else
-        reduce_range<Tag, true>(src, acc, lo, hi, chunk16, seg_stride16, threadIdx.x, blockDim.x);
+        reduce_range<Tag, true, false>(src, acc, lo, hi, chunk16, seg_stride16, threadIdx.x, blockDim.x);
 }
 
 // One launch for all groups.  The work is cut into items (group g, slice s of
 // that group's contiguous range); workgroup b owns items b, b+nb, b+2nb, ...
-// in ascending order, so different workgroups wait on different groups at the
-// same time and many small groups are consumed in parallel.  For its item a
-// workgroup has one lane poll MM[g] == cseg[g] (relaxed agent-scope loads, s_sleep
-// between polls, one acquire fence on success) and then all lanes reduce the slice.  No workgroup waits for
-// another one; the last workgroup to leave resets every group counter (the
-// CAS-to-zero of src/wait.cuh:5-9, deferred to the end of the launch, before
-// which nothing can signal again) and clears workspace word 0.  Word 1 is set
-// if a bounded poll gave up.
+// in ascending order.  With as many slices as workgroups every workgroup takes
+// its slice of every group in turn (large groups: the whole grid works on the
+// group that just completed); with fewer, different workgroups wait on
+// different groups at the same time (many small groups are consumed in
+// parallel).  For its item a workgroup has one lane poll MM[g] == cseg[g]
+// (relaxed agent-scope loads) and then all lanes reduce the slice, reading C
+// past the caches.  There is no acquire fence and no kernel boundary between
+// the groups: either would invalidate the L2 under the running GEMM.
+//
+// A poll is not free for the GEMM running beside the pollers: measured on
+// MI355X, every agent-scope poll costs the 8192^3 GEMM about a nanosecond,
+// wherever the polled word lives (one shared counter or one word per
+// workgroup), so 256 workgroups polling every half microsecond make it 1.7x
+// slower.  The host therefore passes the pause between a lane's polls
+// (sleep_ticks, in s_sleep 16 units of 1024 clocks) so that the launch as a
+// whole stays near ten million polls per second.
+//
+// No workgroup waits for another one; the last workgroup to leave resets every
+// group counter (the CAS-to-zero of src/wait.cuh:5-9, deferred to the end of the
+// launch, before which nothing can signal again) and clears workspace word 0.
+// Word 1 is set if a bounded poll gave up.
 template <typename Tag>
-__global__ __launch_bounds__(CONSUMER_THREADS, 6) void fo_wait_reduce_kernel(
+__global__ __launch_bounds__(CONSUMER_THREADS, 8) void fo_wait_reduce_kernel(
     const fo_u32x4 *C, fo_u32x4 *ACC, int32_t *MM, const int32_t *cseg, int G, long tile16, int W,
-    long seg_stride16, int slices, int32_t *ws, long max_polls) {
+    long seg_stride16, int slices, int32_t *ws, long max_polls, int sleep_ticks) {
     __shared__ int first_tile_s, last;
     const int nb = gridDim.x;
     const long items = (long)G * slices;
@@ -128,27 +163,26 @@ __global__ __launch_bounds__(CONSUMER_THREADS, 6) void fo_wait_reduce_kernel(
                     __hip_atomic_store(ws + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     break;
                 }
-                __builtin_amdgcn_s_sleep(4);
+                for (int k = 0; k < sleep_ticks; k++) __builtin_amdgcn_s_sleep(16);
             }
         }
         __syncthreads();
-        // Polling is relaxed (an acquire per poll would invalidate the L2 under the
-        // running GEMM every time); one acquire per item orders the group's data.
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        // The poll's value has returned before any lane issues a load of the
+        // group's data (barrier above), and those loads do not hit in a cache.
         if (ACC) {
             const long base16 = (long)first_tile_s * tile16;
             const long n16 = (long)cnt * tile16;
             const long lo = n16 * sl / slices, hi = n16 * (sl + 1) / slices;
             if (W <= 1)
-                reduce_range<Tag, false>(C + base16, ACC + base16, lo, hi, 0, 0, threadIdx.x, blockDim.x);
+                reduce_range<Tag, false, true>(C + base16, ACC + base16, lo, hi, 0, 0, threadIdx.x, blockDim.x);
             else
-                reduce_range<Tag, true>(C + base16, ACC + base16 / W, lo, hi, n16 / W, seg_stride16,
-                                        threadIdx.x, blockDim.x);
+                reduce_range<Tag, true, true>(C + base16, ACC + base16 / W, lo, hi, n16 / W, seg_stride16,
+                                              threadIdx.x, blockDim.x);
         }
         __syncthreads();  // first_tile_s is rewritten for the next item
     }
     if (threadIdx.x == 0) {
-        int left = __hip_atomic_fetch_add(ws, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        int left = __hip_atomic_fetch_add(ws, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         last = (left == nb - 1);
     }
     __syncthreads();
@@ -318,28 +352,31 @@ extern "C" int fo_consumer_reduce(int dtype, const void *src, void *acc, int64_t
 
 extern "C" int fo_wait_reduce_groups(int dtype, const void *C, void *ACC, int32_t *MM,
                                      const int32_t *cseg_dev, int G, int64_t tile_elems, int W,
-                                     int64_t seg_stride, int32_t *workspace, int nblocks,
-                                     fo_stream_t stream) {
+                                     int64_t seg_stride, int32_t *workspace, int nblocks, int slices,
+                                     int poll_gap_ns, fo_stream_t stream) {
     if (!MM || !cseg_dev || !workspace || G <= 0 || tile_elems <= 0 || W <= 0) return FO_ERR_ARG;
     if (ACC && !C) return FO_ERR_ARG;
     if (tile_elems % (8 * W) || (W > 1 && seg_stride % 8)) return FO_ERR_SHAPE;
     // The grid spins until the GEMM signals, so it must never be able to crowd the
     // GEMM's workgroups out of every CU: at most one thin workgroup per CU.
     if (nblocks <= 0 || nblocks > CONSUMER_MAX_BLOCKS) nblocks = CONSUMER_MAX_BLOCKS;
-    // Slices per group: enough items to keep every workgroup busy on a large
-    // group, but no slice below one tile's worth of 16-byte pieces.
-    int slices = (nblocks + G - 1) / G;
-    if (slices < 1) slices = 1;
+    if (slices <= 0) slices = (nblocks + G - 1) / G;
+    if (slices > nblocks) slices = nblocks;
+    // pause between one lane's polls: at least what keeps the launch near ten
+    // million polls per second (0.1 us per workgroup), in ticks of about half a microsecond
+    if (poll_gap_ns <= 0) poll_gap_ns = nblocks * 100;
+    int sleep_ticks = (poll_gap_ns + 499) / 500;
+    if (sleep_ticks < 1) sleep_ticks = 1;
     dim3 grid(nblocks), block(CONSUMER_THREADS);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == FO_F16)
         hipLaunchKernelGGL(fo_wait_reduce_kernel<fo_f16_tag>, grid, block, 0, s, (const fo_u32x4 *)C,
                            (fo_u32x4 *)ACC, MM, cseg_dev, G, (long)(tile_elems / 8), W,
-                           (long)(seg_stride / 8), slices, workspace, default_max_polls());
+                           (long)(seg_stride / 8), slices, workspace, default_max_polls(), sleep_ticks);
     else if (dtype == FO_BF16)
         hipLaunchKernelGGL(fo_wait_reduce_kernel<fo_bf16_tag>, grid, block, 0, s, (const fo_u32x4 *)C,
                            (fo_u32x4 *)ACC, MM, cseg_dev, G, (long)(tile_elems / 8), W,
-                           (long)(seg_stride / 8), slices, workspace, default_max_polls());
+                           (long)(seg_stride / 8), slices, workspace, default_max_polls(), sleep_ticks);
     else
         return FO_ERR_DTYPE;
     FO_LAUNCH_CHECK();

@@ -7,18 +7,30 @@ namespace {
 
 using namespace fo_gemm_dev;
 
-// One compiled shape of the kernel template.
+// One compiled shape of the kernel template.  The launch is persistent: as many
+// workgroups as the device keeps resident at once (or fewer, if the problem has
+// fewer macro tiles); each walks the raster with that stride.
 template <typename Tag, int MTM, int MTN, int BK, int STAGES, int WM, int WN, int MODE>
 int launch_variant(const GemmArgs &a, hipStream_t stream) {
     auto kern = fo_gemm_kernel<Tag, MTM, MTN, BK, STAGES, WM, WN, MODE>;
     constexpr int smem = smem_bytes<MTM, MTN, BK, STAGES>();
-    static bool configured = false;  // per instantiation; the attribute is process wide
-    if (!configured) {
+    constexpr int threads = WM * WN * 64;
+    static int resident = 0;  // per instantiation; the attribute is process wide
+    if (!resident) {
         FO_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-        configured = true;
+        int dev = 0, cus = 0, per_cu = 0;
+        FO_HIP_CHECK(hipGetDevice(&dev));
+        FO_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+        FO_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(kern),
+                                                                  threads, smem));
+        if (cus <= 0 || per_cu <= 0) return FO_ERR_STATE;
+        // a multiple of 8 keeps "workgroup id mod 8 = XCD" true for every tile of the walk
+        resident = (cus * per_cu) / 8 * 8;
+        if (resident <= 0) resident = cus * per_cu;
     }
-    dim3 grid(a.grid_m * a.grid_n), block(WM * WN * 64);
+    const int ntiles = a.grid_m * a.grid_n;
+    dim3 grid(ntiles < resident ? ntiles : resident), block(threads);
     hipLaunchKernelGGL(kern, grid, block, smem, stream, a);
     FO_LAUNCH_CHECK();
     return FO_OK;
@@ -54,6 +66,8 @@ int run_gemm(int mode, int dtype, int M, int N, int K, int rLDN, const int32_t *
     int rc = fo_pick_raster(algo, M, N, &r);
     if (rc) return rc;
     if (K % 64) return FO_ERR_SHAPE;
+    // the epilogue assumes a wavefront's 128 x 64 (or 64 x 64) block lies inside one reorder tile
+    if (e->f[0] % 128 || e->f[1] % 128) return FO_ERR_ALGO;
     GemmArgs a;
     a.A = static_cast<const uint16_t *>(A);
     a.B = static_cast<const uint16_t *>(B);

@@ -9,7 +9,7 @@ struct fo_overlap {
     hipStream_t gemm_stream = nullptr;
     hipStream_t comm_stream = nullptr;
     hipEvent_t joined = nullptr;
-    int32_t *workspace = nullptr;  // one zeroed word for the fused wait+reduce kernel
+    int32_t *workspace = nullptr;  // zeroed words of the one-launch wait+reduce kernel
     bool gemm_ready = false;
     bool overlap_ready = false;
     int rank = 0, world = 1;
@@ -21,13 +21,36 @@ struct fo_overlap {
 namespace {
 
 // Two launches per group cost a few microseconds each; beyond this many groups
-// the single wait+reduce launch is the faster consumer.
+// the single wait+reduce launch is the faster consumer.  With few, large groups
+// the per-group launches win: a kernel that starts when its group is complete
+// needs no polling workgroups resident beside the GEMM.
 constexpr int kFusedFromGroups = 16;
 
 int fused_grid(const fo_overlap *h, int G) {  // 0: per-group launches, otherwise workgroups of the one launch
     if (h->fused < 0) return G > kFusedFromGroups ? 256 : 0;
     if (h->fused == 1) return 256;
     return h->fused;
+}
+
+// Pause between a workgroup's polls in the one-launch consumer: 100 ns per
+// workgroup keeps the GEMM's slowdown near one percent, but no more than about
+// a sixtieth of the GEMM's expected duration (at 1.2 PFLOP/s), so that a short
+// problem is not left waiting for a sleeping poller.
+int fused_poll_gap_ns(int M, int N, int K, int grid) {
+    const double gemm_ns = 2.0 * M * N * K / 1.2e6;
+    double gap = grid * 100.0;
+    if (gap > gemm_ns / 60) gap = gemm_ns / 60;
+    if (gap < 500) gap = 500;
+    return (int)gap;
+}
+
+// Pieces per group for the one-launch consumer: about 32 KiB each, at most one per workgroup.
+int fused_slices(int64_t total_elems, int G, int grid) {
+    const int64_t per_group = total_elems / G;
+    int64_t s = per_group / 16384;
+    if (s < 1) s = 1;
+    if (s > grid) s = grid;
+    return (int)s;
 }
 
 int check_segments(const int32_t *cseg_host, int G, long tiles) {
@@ -142,7 +165,8 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
     const int fused = fused_grid(h, G);
     if (fused) {
         rc = fo_wait_reduce_groups(dtype, C, h->acc, MM, cseg_dev, G, tile_elems, 1, 0, h->workspace,
-                                   fused, h->comm_stream);
+                                   fused, fused_slices((int64_t)M * N, G, fused),
+                                   fused_poll_gap_ns(M, N, K, fused), h->comm_stream);
         if (rc) return rc;
     } else {
         int64_t off = 0;
@@ -192,7 +216,8 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
     const int fused = fused_grid(h, G);
     if (fused) {
         rc = fo_wait_reduce_groups(dtype, C, h->acc, MM, cseg_dev, G, tile_elems, W, seg_stride,
-                                   h->workspace, fused, h->comm_stream);
+                                   h->workspace, fused, fused_slices((int64_t)M * N, G, fused),
+                                   fused_poll_gap_ns(M, N, K, fused), h->comm_stream);
         if (rc) return rc;
     }
     int64_t off = 0;

@@ -96,11 +96,11 @@ def consumer_reduce_rs(src, acc, W, seg_stride, stream=None):
 
 
 def wait_reduce_groups(C, ACC, MM, cseg_dev, tile_elems, workspace, W=1, seg_stride=0, nblocks=0,
-                       stream=None):
+                       slices=0, poll_gap_ns=0, stream=None):
     check(lib().fo_wait_reduce_groups(dtype_code(C), _ptr(C, "C"), _ptr(ACC, "ACC"), _i32(MM, "MM"),
                                       _i32(cseg_dev, "cSeg"), cseg_dev.numel(), int(tile_elems),
                                       int(W), int(seg_stride), _i32(workspace, "workspace"),
-                                      int(nblocks), _stream(stream)), "fo_wait_reduce_groups")
+                                      int(nblocks), int(slices), int(poll_gap_ns), _stream(stream)), "fo_wait_reduce_groups")
 
 
 def reorder_rmsnorm(X, Y, Wt, BM, BN, rldn, RA, eps=1e-5, stream=None):

@@ -128,11 +128,20 @@ int fo_consumer_reduce_rs(int dtype, const void *src, void *acc, int64_t nelem, 
  * The counters are reset by the last workgroup to leave instead of per group.
  * workspace: device int32[2], zero before the first use; the kernel leaves
  * word 0 zero and sets word 1 only if a bounded poll gave up (see
- * FO_WAIT_MAX_POLLS below).  nblocks <= 0 picks a default. */
+ * FO_WAIT_MAX_POLLS below).  nblocks <= 0 picks a default grid.  slices = into
+ * how many pieces a group's range is cut (one piece per workgroup at a time):
+ * nblocks for large groups, so that the whole grid consumes the group that
+ * just completed; fewer for small groups, so that different workgroups serve
+ * different groups; <= 0 picks ceil(nblocks / G).  poll_gap_ns = pause between
+ * one workgroup's polls of its group counter; every poll slows a GEMM running
+ * beside the kernel a little, so <= 0 picks 100 ns per workgroup (about ten
+ * million polls per second in total); pass less for problems that are over
+ * in tens of microseconds.  C is read past the caches and the kernel contains
+ * no acquire fence, so it does not disturb the L2 of a GEMM running beside it. */
 int fo_wait_reduce_groups(int dtype, const void *C, void *ACC, int32_t *MM,
                           const int32_t *cseg_dev, int G, int64_t tile_elems, int W,
-                          int64_t seg_stride, int32_t *workspace, int nblocks,
-                          fo_stream_t stream);
+                          int64_t seg_stride, int32_t *workspace, int nblocks, int slices,
+                          int poll_gap_ns, fo_stream_t stream);
 
 /* ---- RMSNorm ----------------------------------------------------------
  * Replaces reorder_rmsnorm(X, RX, RW, BM, BN, rldn, RA), src/rmsnorm/rmsnorm.h:6-8,
@@ -168,9 +177,9 @@ int fo_overlap_set_world(fo_overlap_t *h, int rank, int world);
  * [W, M/W, N] (seg_stride = M/W*N elements). */
 int fo_overlap_set_accumulator(fo_overlap_t *h, void *acc, int64_t nelem);
 /* fused < 0 (default): chosen per call, one launch when there are more than 16
- * groups; 0: always 2*G launches as the reference's host loop; 1: always one
- * fo_wait_reduce_groups launch with the default grid; n > 1: the same with n
- * workgroups. */
+ * groups; 0: always 2*G launches as the reference's host loop
+ * (src/overlap_impl.cu:250-258); 1: always one fo_wait_reduce_groups launch
+ * with the default grid; n > 1: the same with n workgroups. */
 int fo_overlap_set_fused_consumer(fo_overlap_t *h, int fused);
 fo_stream_t fo_overlap_comm_stream(fo_overlap_t *h);
 
