@@ -66,10 +66,7 @@ __device__ __forceinline__ fo_u32x4 load16_coherent(const fo_u32x4 *base, unsign
 
 // dst[i] += src[i] for i in [lo, hi) (16-byte units), the workgroup's lanes striding together.
 // RS: piece i belongs to chunk q = i / chunk16 and lands at dst + q*seg_stride16 + (i - q*chunk16).
-// COHERENT: src is read past the caches (see load16_coherent).  Everything else is
-// streamed with the non-temporal cache policy: the data is touched once, and
-// lines kept for it would push the operand panels of a GEMM running beside the
-// consumer out of the L2.
+// COHERENT: src is read past the caches (see load16_coherent).
 template <typename Tag, bool RS, bool COHERENT>
 __device__ __forceinline__ void reduce_range(const fo_u32x4 *src, fo_u32x4 *dst, long lo, long hi,
                                              long chunk16, long seg_stride16, int tid, int nthreads) {
@@ -80,7 +77,7 @@ __device__ __forceinline__ void reduce_range(const fo_u32x4 *src, fo_u32x4 *dst,
     };
     auto fetch = [&](long first, int u) -> fo_u32x4 {  // src[first + tid + u * nthreads], first wave-uniform
         if (COHERENT) return load16_coherent(src + first, (unsigned)(tid + u * nthreads) * 16u);
-        return __builtin_nontemporal_load(src + first + tid + (long)u * nthreads);
+        return src[first + tid + (long)u * nthreads];
     };
     constexpr int U = RS ? CONSUMER_UNROLL / 2 : CONSUMER_UNROLL;
     long first = lo;
@@ -91,14 +88,14 @@ __device__ __forceinline__ void reduce_range(const fo_u32x4 *src, fo_u32x4 *dst,
 #pragma unroll
         for (int u = 0; u < U; u++) a[u] = fetch(first, u);
 #pragma unroll
-        for (int u = 0; u < U; u++) b[u] = __builtin_nontemporal_load(where(i + (long)u * nthreads));
+        for (int u = 0; u < U; u++) b[u] = *where(i + (long)u * nthreads);
 #pragma unroll
-        for (int u = 0; u < U; u++) __builtin_nontemporal_store(add8<Tag>(b[u], a[u]), where(i + (long)u * nthreads));
+        for (int u = 0; u < U; u++) *where(i + (long)u * nthreads) = add8<Tag>(b[u], a[u]);
     }
     for (; first < hi; first += nthreads) {
         if (first + tid < hi) {
             fo_u32x4 *d = where(first + tid);
-            __builtin_nontemporal_store(add8<Tag>(__builtin_nontemporal_load(d), fetch(first, 0)), d);
+            *d = add8<Tag>(*d, fetch(first, 0));
         }
     }
 }

@@ -153,7 +153,7 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
     constexpr int STAGE16 = (MTM + MTN) * CH;                    // stage size in 16-byte units
     constexpr int KK = BK / 16;                                  // MFMA k-steps per stage
     constexpr int NM = FM * FN, NR = FM + FN;
-    // epilogue: per-wavefront strip of 32 rows x WTN columns in the last ring slot
+    // epilogue: per-wavefront strip of 32 rows x WTN columns in the ring behind slot 0
     constexpr int PITCH = WTN + 8;   // halfs; keeps 16-byte alignment, skews banks
     constexpr int CPR = WTN / 8;     // 16-byte chunks per strip row
     constexpr int RPP = 64 / CPR;    // strip rows per store pass
@@ -162,7 +162,7 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
     static_assert(A_BLK % NW == 0 && B_BLK % NW == 0, "tile rows must split evenly over the wavefronts");
     static_assert((NW * (64 / CH)) % 32 == 0, "swizzle key must repeat across a wavefront's blocks");
     static_assert(STAGES >= 2, "ring depth");
-    static_assert(NW * 32 * PITCH * 2 <= STAGE16 * 16, "the epilogue strips must fit into one ring slot");
+    static_assert(NW * 32 * PITCH * 2 <= (STAGES - 1) * STAGE16 * 16, "the epilogue strips must fit behind ring slot 0");
     static_assert((STAGES - 1) * P + NST < 64, "vmcnt range");
 
     extern __shared__ fo_u32x4 smem[];
@@ -359,7 +359,7 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
 
         // Stage 0 of this tile is in flight.  First tile: request the rest of the
         // ring, then wait for stage 0.  Later tiles: stage 0 was requested before
-        // the previous epilogue, whose strips lived in the last slot, so the rest
+        // the previous epilogue, whose strips lived behind slot 0, so the rest
         // of the ring is requested only after the barrier; the previous tile's
         // NST stores are younger than stage 0 and need not have completed.
         if (!carried) {
@@ -437,7 +437,7 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
             int el = lane;
             asm volatile("" : "+v"(el));
             const int erow = el & 31, ek = el >> 5;
-            uint16_t *strip = reinterpret_cast<uint16_t *>(smem + (STAGES - 1) * STAGE16) + wave * (32 * PITCH);
+            uint16_t *strip = reinterpret_cast<uint16_t *>(smem + STAGE16) + wave * (32 * PITCH);
             const int srow = el / CPR, scol = el % CPR;
             const int ldp = MODE == MODE_PLAIN ? p.N : p.rLDN * p.BN;  // leading dimension of the output view
             const int row0 = (wm * WTM) % p.BM, col0 = (wn * WTN) % p.BN;  // of this wavefront inside its reorder tile

@@ -117,6 +117,20 @@ def test_signal_gemm_many_groups_and_rldn(fo, oracle):
     _signal_case(fo, oracle, F16, 128, 128, 512, 512, 64, [16], rldn=4)
 
 
+def test_signal_gemm_persistent_walk(fo, oracle):
+    """More tiles than resident workgroups: some workgroups compute several tiles, request
+    the next tile's operands before their epilogue and send the previous tile's signal late."""
+    # 600 tiles of 128x128 (M is no multiple of 256, so the workgroup tile is 128x128; 512 are resident)
+    _signal_case(fo, oracle, F16, 128, 128, 3200, 3072, 128, [100] * 6)
+    # one K step per tile: the signal cannot ride in the next tile's K loop and is sent at once
+    _signal_case(fo, oracle, BF16, 128, 128, 3200, 3072, 64, [599, 1])
+    # 272 workgroup tiles of 256x256 on 256 resident workgroups, four reorder tiles each
+    _signal_case(fo, oracle, F16, 128, 128, 4352, 4096, 128, [272] * 4, swizzle=4)
+    _signal_case(fo, oracle, F16, 256, 128, 4352, 4096, 192, [300, 244], swizzle=4, W=2)
+    # 1089 groups: beyond the group table kept in LDS, the lookup scans cSeg in memory
+    _signal_case(fo, oracle, F16, 128, 128, 4224, 4224, 64, [1] * 1089)
+
+
 def test_scatter_gemm_row_map(fo, oracle):
     _signal_case(fo, oracle, F16, 128, 128, 512, 512, 64, [4, 4, 8], W=4)
     _signal_case(fo, oracle, BF16, 128, 128, 512, 256, 128, [3, 5], W=8)
