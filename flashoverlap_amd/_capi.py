@@ -21,6 +21,8 @@ SIGNATURES = {
     "fo_algo_info": (c_int, [c_int, vp]),
     "fo_schedule_order": (c_int, [c_int, c_int, c_int, vp]),
     "fo_workgroup_tiles": (c_int, [c_int, c_int, c_int, vp, vp]),
+    "fo_gemm_wave_tiles": (c_int, [c_int, c_int, c_int, c_int, vp]),
+    "fo_wait_groups": (c_int, [c_int, vp, vp, vp]),
     "fo_gemm": (c_int, [c_int, c_int, c_int, c_int, vp, vp, vp, c_int, vp]),
     "fo_gemm_signal": (c_int, [c_int, c_int, c_int, c_int, c_int, vp, c_int, vp, vp, vp, vp, vp,
                                c_int, c_int, vp]),
@@ -30,8 +32,9 @@ SIGNATURES = {
     "fo_wait_bounded": (c_int, [c_int, vp, c_i64, vp, vp]),
     "fo_consumer_reduce": (c_int, [c_int, vp, vp, c_i64, vp]),
     "fo_consumer_reduce_rs": (c_int, [c_int, vp, vp, c_i64, c_int, c_i64, vp]),
-    "fo_wait_reduce_groups": (c_int, [c_int, vp, vp, vp, vp, c_int, c_i64, c_int, c_i64, vp, c_int,
-                                      c_int, c_int, vp]),
+    "fo_consumer_reduce_rs_own": (c_int, [c_int, vp, vp, c_i64, c_int, c_i64, vp, c_int, vp]),
+    "fo_wait_reduce_groups": (c_int, [c_int, vp, vp, vp, vp, c_int, c_i64, c_int, c_i64, vp, c_int, vp,
+                                      c_int, c_int, c_int, vp]),
     "fo_reorder_rmsnorm": (c_int, [c_int, vp, vp, vp, c_int, c_int, c_int, c_int, c_int, vp, c_f32,
                                    vp]),
     "fo_rmsnorm": (c_int, [c_int, vp, vp, vp, c_int, c_int, c_f32, vp]),
@@ -119,9 +122,9 @@ def schedule_order(algo, M, N):
     return list(buf)
 
 
-def wave_tiles(algo, M, N, cus=256):
-    """Reorder tiles one wave of the chip completes: CUs x tiles per workgroup."""
-    per = ctypes.c_int32()
-    wgs = ctypes.c_int32()
-    check(lib().fo_workgroup_tiles(int(algo), M, N, ctypes.byref(per), ctypes.byref(wgs)), "fo_workgroup_tiles")
-    return cus * per.value
+def wave_tiles(algo, M, N, dtype=F16):
+    """Reorder tiles that complete together: resident workgroups of the persistent
+    GEMM x reorder tiles per workgroup (asks the GPU for the kernel's occupancy)."""
+    tiles = ctypes.c_int32()
+    check(lib().fo_gemm_wave_tiles(int(dtype), int(algo), M, N, ctypes.byref(tiles)), "fo_gemm_wave_tiles")
+    return tiles.value

@@ -29,6 +29,25 @@ __global__ void fo_wait_kernel(int expect, int32_t *counter, long max_polls, int
     }
 }
 
+// The same for `count` consecutive groups, one after the other.
+__global__ void fo_wait_groups_kernel(int count, const int32_t *expect, int32_t *counters, long max_polls) {
+    for (int g = 0; g < count; g++) {
+        const int want = expect[g];
+        long polls = 0;
+        for (;;) {
+            int v = __hip_atomic_load(counters + g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (v == want) {
+                int e = want;
+                if (__hip_atomic_compare_exchange_strong(counters + g, &e, 0, __ATOMIC_ACQ_REL, __ATOMIC_RELAXED,
+                                                         __HIP_MEMORY_SCOPE_AGENT))
+                    break;
+            }
+            if (max_polls > 0 && ++polls >= max_polls) return;
+            __builtin_amdgcn_s_sleep(8);
+        }
+    }
+}
+
 // ------------------------------------------------------------------ consumer
 template <typename Tag>
 __device__ __forceinline__ fo_u32x4 add8(fo_u32x4 a, fo_u32x4 b) {
@@ -66,14 +85,23 @@ __device__ __forceinline__ fo_u32x4 load16_coherent(const fo_u32x4 *base, unsign
 
 // dst[i] += src[i] for i in [lo, hi) (16-byte units), the workgroup's lanes striding together.
 // RS: piece i belongs to chunk q = i / chunk16 and lands at dst + q*seg_stride16 + (i - q*chunk16).
+// With `own` set, the pieces of chunk `rank` are also copied to own + (i - rank*chunk16): this
+// rank's share of the group, the output of a reduce-scatter with one rank present.
 // COHERENT: src is read past the caches (see load16_coherent).
 template <typename Tag, bool RS, bool COHERENT>
 __device__ __forceinline__ void reduce_range(const fo_u32x4 *src, fo_u32x4 *dst, long lo, long hi,
-                                             long chunk16, long seg_stride16, int tid, int nthreads) {
+                                             long chunk16, long seg_stride16, int tid, int nthreads,
+                                             fo_u32x4 *own = nullptr, int rank = 0) {
     auto where = [&](long k) -> fo_u32x4 * {
         if (!RS) return dst + k;
         const long q = k / chunk16;
         return dst + q * seg_stride16 + (k - q * chunk16);
+    };
+    auto keep = [&](long k, fo_u32x4 v) {
+        if (RS && own) {
+            const long r = k - (long)rank * chunk16;
+            if (r >= 0 && r < chunk16) own[r] = v;
+        }
     };
     auto fetch = [&](long first, int u) -> fo_u32x4 {  // src[first + tid + u * nthreads], first wave-uniform
         if (COHERENT) return load16_coherent(src + first, (unsigned)(tid + u * nthreads) * 16u);
@@ -91,11 +119,15 @@ __device__ __forceinline__ void reduce_range(const fo_u32x4 *src, fo_u32x4 *dst,
         for (int u = 0; u < U; u++) b[u] = *where(i + (long)u * nthreads);
 #pragma unroll
         for (int u = 0; u < U; u++) *where(i + (long)u * nthreads) = add8<Tag>(b[u], a[u]);
+#pragma unroll
+        for (int u = 0; u < U; u++) keep(i + (long)u * nthreads, a[u]);
     }
     for (; first < hi; first += nthreads) {
         if (first + tid < hi) {
             fo_u32x4 *d = where(first + tid);
-            *d = add8<Tag>(*d, fetch(first, 0));
+            const fo_u32x4 a = fetch(first, 0);
+            *d = add8<Tag>(*d, a);
+            keep(first + tid, a);
         }
     }
 }
@@ -104,7 +136,8 @@ __device__ __forceinline__ void reduce_range(const fo_u32x4 *src, fo_u32x4 *dst,
 template <typename Tag>
 __global__ __launch_bounds__(CONSUMER_THREADS, 8) void fo_consumer_kernel(const fo_u32x4 *src, fo_u32x4 *acc,
                                                                        long chunk16, int W,
-                                                                       long seg_stride16) {
+                                                                       long seg_stride16, fo_u32x4 *own,
+                                                                       int rank) {
     const long total = chunk16 * W;
     const long per = (total + gridDim.x - 1) / gridDim.x;
     const long lo = per * blockIdx.x;
@@ -113,7 +146,8 @@ __global__ __launch_bounds__(CONSUMER_THREADS, 8) void fo_consumer_kernel(const 
     if (W <= 1)
         reduce_range<Tag, false, false>(src, acc, lo, hi, 0, 0, threadIdx.x, blockDim.x);
     else
-        reduce_range<Tag, true, false>(src, acc, lo, hi, chunk16, seg_stride16, threadIdx.x, blockDim.x);
+        reduce_range<Tag, true, false>(src, acc, lo, hi, chunk16, seg_stride16, threadIdx.x, blockDim.x, own,
+                                       rank);
 }
 
 // One launch for all groups.  The work is cut into items (group g, slice s of
@@ -142,7 +176,7 @@ __global__ __launch_bounds__(CONSUMER_THREADS, 8) void fo_consumer_kernel(const 
 template <typename Tag>
 __global__ __launch_bounds__(CONSUMER_THREADS, 8) void fo_wait_reduce_kernel(
     const fo_u32x4 *C, fo_u32x4 *ACC, int32_t *MM, const int32_t *cseg, int G, long tile16, int W,
-    long seg_stride16, int slices, int32_t *ws, long max_polls, int sleep_ticks) {
+    long seg_stride16, int slices, int32_t *ws, long max_polls, int sleep_ticks, fo_u32x4 *OWN, int rank) {
     __shared__ int first_tile_s, last;
     const int nb = gridDim.x;
     const long items = (long)G * slices;
@@ -174,7 +208,7 @@ __global__ __launch_bounds__(CONSUMER_THREADS, 8) void fo_wait_reduce_kernel(
                 reduce_range<Tag, false, true>(C + base16, ACC + base16, lo, hi, 0, 0, threadIdx.x, blockDim.x);
             else
                 reduce_range<Tag, true, true>(C + base16, ACC + base16 / W, lo, hi, n16 / W, seg_stride16,
-                                              threadIdx.x, blockDim.x);
+                                              threadIdx.x, blockDim.x, OWN ? OWN + base16 / W : nullptr, rank);
         }
         __syncthreads();  // first_tile_s is rewritten for the next item
     }
@@ -312,6 +346,14 @@ extern "C" int fo_wait(int expect, int32_t *counter, fo_stream_t stream) {
     return FO_OK;
 }
 
+extern "C" int fo_wait_groups(int count, const int32_t *expect_dev, int32_t *counters, fo_stream_t stream) {
+    if (count <= 0 || !expect_dev || !counters) return FO_ERR_ARG;
+    hipLaunchKernelGGL(fo_wait_groups_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream), count,
+                       expect_dev, counters, default_max_polls());
+    FO_LAUNCH_CHECK();
+    return FO_OK;
+}
+
 extern "C" int fo_wait_bounded(int expect, int32_t *counter, int64_t max_polls, int32_t *status,
                                fo_stream_t stream) {
     if (!counter || max_polls < 0) return FO_ERR_ARG;
@@ -321,25 +363,36 @@ extern "C" int fo_wait_bounded(int expect, int32_t *counter, int64_t max_polls, 
     return FO_OK;
 }
 
-extern "C" int fo_consumer_reduce_rs(int dtype, const void *src, void *acc, int64_t nelem, int W,
-                                     int64_t seg_stride, fo_stream_t stream) {
+extern "C" int fo_consumer_reduce_rs_own(int dtype, const void *src, void *acc, int64_t nelem, int W,
+                                         int64_t seg_stride, void *own, int rank, fo_stream_t stream) {
     if (!src || !acc || nelem < 0 || W <= 0) return FO_ERR_ARG;
+    if (own && (rank < 0 || rank >= W)) return FO_ERR_ARG;
     if (nelem == 0) return FO_OK;
     if (nelem % W || (nelem / W) % 8 || (W > 1 && seg_stride % 8)) return FO_ERR_SHAPE;
-    if (((uintptr_t)src | (uintptr_t)acc) & 15) return FO_ERR_SHAPE;
+    if (((uintptr_t)src | (uintptr_t)acc | (uintptr_t)own) & 15) return FO_ERR_SHAPE;
     const long chunk16 = nelem / W / 8;
+    if (own && W == 1) {  // the whole range is this rank's: a plain copy beside the reduce
+        FO_HIP_CHECK(hipMemcpyAsync(own, src, (size_t)nelem * 2, hipMemcpyDeviceToDevice,
+                                    static_cast<hipStream_t>(stream)));
+        own = nullptr;
+    }
     dim3 grid(consumer_grid(chunk16 * W)), block(CONSUMER_THREADS);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == FO_F16)
         hipLaunchKernelGGL(fo_consumer_kernel<fo_f16_tag>, grid, block, 0, s, (const fo_u32x4 *)src,
-                           (fo_u32x4 *)acc, chunk16, W, (long)(seg_stride / 8));
+                           (fo_u32x4 *)acc, chunk16, W, (long)(seg_stride / 8), (fo_u32x4 *)own, rank);
     else if (dtype == FO_BF16)
         hipLaunchKernelGGL(fo_consumer_kernel<fo_bf16_tag>, grid, block, 0, s, (const fo_u32x4 *)src,
-                           (fo_u32x4 *)acc, chunk16, W, (long)(seg_stride / 8));
+                           (fo_u32x4 *)acc, chunk16, W, (long)(seg_stride / 8), (fo_u32x4 *)own, rank);
     else
         return FO_ERR_DTYPE;
     FO_LAUNCH_CHECK();
     return FO_OK;
+}
+
+extern "C" int fo_consumer_reduce_rs(int dtype, const void *src, void *acc, int64_t nelem, int W,
+                                     int64_t seg_stride, fo_stream_t stream) {
+    return fo_consumer_reduce_rs_own(dtype, src, acc, nelem, W, seg_stride, nullptr, 0, stream);
 }
 
 extern "C" int fo_consumer_reduce(int dtype, const void *src, void *acc, int64_t nelem,
@@ -349,10 +402,11 @@ extern "C" int fo_consumer_reduce(int dtype, const void *src, void *acc, int64_t
 
 extern "C" int fo_wait_reduce_groups(int dtype, const void *C, void *ACC, int32_t *MM,
                                      const int32_t *cseg_dev, int G, int64_t tile_elems, int W,
-                                     int64_t seg_stride, int32_t *workspace, int nblocks, int slices,
-                                     int poll_gap_ns, fo_stream_t stream) {
+                                     int64_t seg_stride, void *own, int rank, int32_t *workspace,
+                                     int nblocks, int slices, int poll_gap_ns, fo_stream_t stream) {
     if (!MM || !cseg_dev || !workspace || G <= 0 || tile_elems <= 0 || W <= 0) return FO_ERR_ARG;
     if (ACC && !C) return FO_ERR_ARG;
+    if (own && (!ACC || W < 2 || rank < 0 || rank >= W)) return FO_ERR_ARG;
     if (tile_elems % (8 * W) || (W > 1 && seg_stride % 8)) return FO_ERR_SHAPE;
     // The grid spins until the GEMM signals, so it must never be able to crowd the
     // GEMM's workgroups out of every CU: at most one thin workgroup per CU.
@@ -369,11 +423,13 @@ extern "C" int fo_wait_reduce_groups(int dtype, const void *C, void *ACC, int32_
     if (dtype == FO_F16)
         hipLaunchKernelGGL(fo_wait_reduce_kernel<fo_f16_tag>, grid, block, 0, s, (const fo_u32x4 *)C,
                            (fo_u32x4 *)ACC, MM, cseg_dev, G, (long)(tile_elems / 8), W,
-                           (long)(seg_stride / 8), slices, workspace, default_max_polls(), sleep_ticks);
+                           (long)(seg_stride / 8), slices, workspace, default_max_polls(), sleep_ticks,
+                           (fo_u32x4 *)own, rank);
     else if (dtype == FO_BF16)
         hipLaunchKernelGGL(fo_wait_reduce_kernel<fo_bf16_tag>, grid, block, 0, s, (const fo_u32x4 *)C,
                            (fo_u32x4 *)ACC, MM, cseg_dev, G, (long)(tile_elems / 8), W,
-                           (long)(seg_stride / 8), slices, workspace, default_max_polls(), sleep_ticks);
+                           (long)(seg_stride / 8), slices, workspace, default_max_polls(), sleep_ticks,
+                           (fo_u32x4 *)own, rank);
     else
         return FO_ERR_DTYPE;
     FO_LAUNCH_CHECK();

@@ -10,8 +10,10 @@ using namespace fo_gemm_dev;
 // One compiled shape of the kernel template.  The launch is persistent: as many
 // workgroups as the device keeps resident at once (or fewer, if the problem has
 // fewer macro tiles); each walks the raster with that stride.
+// With `resident_out` set nothing is launched: the call only reports how many workgroups the
+// launch would hold.
 template <typename Tag, int MTM, int MTN, int BK, int STAGES, int WM, int WN, int MODE>
-int launch_variant(const GemmArgs &a, hipStream_t stream) {
+int launch_variant(const GemmArgs &a, hipStream_t stream, int *resident_out) {
     auto kern = fo_gemm_kernel<Tag, MTM, MTN, BK, STAGES, WM, WN, MODE>;
     constexpr int smem = smem_bytes<MTM, MTN, BK, STAGES>();
     constexpr int threads = WM * WN * 64;
@@ -30,6 +32,10 @@ int launch_variant(const GemmArgs &a, hipStream_t stream) {
         if (resident <= 0) resident = cus * per_cu;
     }
     const int ntiles = a.grid_m * a.grid_n;
+    if (resident_out) {
+        *resident_out = ntiles < resident ? ntiles : resident;
+        return FO_OK;
+    }
     dim3 grid(ntiles < resident ? ntiles : resident), block(threads);
     hipLaunchKernelGGL(kern, grid, block, smem, stream, a);
     FO_LAUNCH_CHECK();
@@ -40,18 +46,22 @@ int launch_variant(const GemmArgs &a, hipStream_t stream) {
 // 64 KiB) is the workhorse; the smaller shapes serve problems whose M or N is
 // not a multiple of 256 or that have too few 256x256 tiles to fill the chip.
 template <typename Tag, int MODE>
-int launch_tile(const GemmArgs &a, int mtm, int mtn, hipStream_t stream) {
-    if (mtm == 256 && mtn == 256) return launch_variant<Tag, 256, 256, 64, 2, 2, 4, MODE>(a, stream);
-    if (mtm == 128 && mtn == 128) return launch_variant<Tag, 128, 128, 64, 2, 2, 2, MODE>(a, stream);
-    if (mtm == 128 && mtn == 256) return launch_variant<Tag, 128, 256, 64, 3, 2, 4, MODE>(a, stream);
-    if (mtm == 256 && mtn == 128) return launch_variant<Tag, 256, 128, 64, 3, 2, 2, MODE>(a, stream);
+int launch_tile(const GemmArgs &a, int mtm, int mtn, hipStream_t stream, int *resident_out) {
+    if (mtm == 256 && mtn == 256)
+        return launch_variant<Tag, 256, 256, 64, 2, 2, 4, MODE>(a, stream, resident_out);
+    if (mtm == 128 && mtn == 128)
+        return launch_variant<Tag, 128, 128, 64, 2, 2, 2, MODE>(a, stream, resident_out);
+    if (mtm == 128 && mtn == 256)
+        return launch_variant<Tag, 128, 256, 64, 3, 2, 4, MODE>(a, stream, resident_out);
+    if (mtm == 256 && mtn == 128)
+        return launch_variant<Tag, 256, 128, 64, 3, 2, 2, MODE>(a, stream, resident_out);
     return FO_ERR_ALGO;
 }
 
 template <int MODE>
-int launch_dtype(int dtype, const GemmArgs &a, int mtm, int mtn, hipStream_t stream) {
-    if (dtype == FO_F16) return launch_tile<fo_f16_tag, MODE>(a, mtm, mtn, stream);
-    if (dtype == FO_BF16) return launch_tile<fo_bf16_tag, MODE>(a, mtm, mtn, stream);
+int launch_dtype(int dtype, const GemmArgs &a, int mtm, int mtn, hipStream_t stream, int *resident_out = nullptr) {
+    if (dtype == FO_F16) return launch_tile<fo_f16_tag, MODE>(a, mtm, mtn, stream, resident_out);
+    if (dtype == FO_BF16) return launch_tile<fo_bf16_tag, MODE>(a, mtm, mtn, stream, resident_out);
     return FO_ERR_DTYPE;
 }
 
@@ -96,6 +106,23 @@ int run_gemm(int mode, int dtype, int M, int N, int K, int rLDN, const int32_t *
 }
 
 }  // namespace
+
+extern "C" int fo_gemm_wave_tiles(int dtype, int algo, int M, int N, int32_t *tiles) {
+    if (!tiles) return FO_ERR_ARG;
+    const fo_algo_entry *e = fo_algo_lookup(algo);
+    if (!e) return FO_ERR_ALGO;
+    fo_raster r;
+    int rc = fo_pick_raster(algo, M, N, &r);
+    if (rc) return rc;
+    GemmArgs a = {};
+    a.grid_m = r.grid_m;
+    a.grid_n = r.grid_n;
+    int resident = 0;
+    rc = launch_dtype<MODE_SIGNAL>(dtype, a, r.mtm, r.mtn, nullptr, &resident);
+    if (rc) return rc;
+    *tiles = resident * (r.mtm / e->f[0]) * (r.mtn / e->f[1]);
+    return FO_OK;
+}
 
 extern "C" int fo_gemm(int dtype, int M, int N, int K, const void *A, const void *B, void *C,
                        int algo, fo_stream_t stream) {

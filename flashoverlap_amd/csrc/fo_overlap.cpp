@@ -53,6 +53,20 @@ int fused_slices(int64_t total_elems, int G, int grid) {
     return (int)s;
 }
 
+// Groups [i, j) that complete in the same wave of the persistent GEMM (their last
+// tiles fall into the same stretch of `wave` consecutive storage slots, which
+// is the order the hint assigns) are waited for by one launch: they become
+// ready within microseconds of each other, and a launch per group would only
+// add its latency to the tail.  done = tiles of the groups before i.
+int batch_end(const int32_t *cseg_host, int G, int i, long done, int wave) {
+    if (wave <= 0) return i + 1;
+    const long w = (done + cseg_host[i] - 1) / wave;
+    int j = i + 1;
+    long d = done + cseg_host[i];
+    while (j < G && (d + cseg_host[j] - 1) / wave == w) d += cseg_host[j++];
+    return j;
+}
+
 int check_segments(const int32_t *cseg_host, int G, long tiles) {
     if (!cseg_host || G <= 0) return FO_ERR_SEGMENTS;
     long sum = 0;
@@ -158,29 +172,41 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
     const int64_t tile_elems = (int64_t)info[0] * info[1];
     if (h->acc && h->acc_nelem < (int64_t)M * N) return FO_ERR_ARG;
 
+    const int fused = fused_grid(h, G);
+    int32_t wave = 0;
+    if (!fused) {
+        rc = fo_gemm_wave_tiles(dtype, algo, M, N, &wave);
+        if (rc) return rc;
+    }
     rc = fo_gemm_signal(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, MM, RA, monitor, algo,
                         h->gemm_stream);
     if (rc) return rc;  // nothing has been enqueued on the consumer stream yet
 
-    const int fused = fused_grid(h, G);
     if (fused) {
-        rc = fo_wait_reduce_groups(dtype, C, h->acc, MM, cseg_dev, G, tile_elems, 1, 0, h->workspace,
-                                   fused, fused_slices((int64_t)M * N, G, fused),
+        rc = fo_wait_reduce_groups(dtype, C, h->acc, MM, cseg_dev, G, tile_elems, 1, 0, nullptr, 0,
+                                   h->workspace, fused, fused_slices((int64_t)M * N, G, fused),
                                    fused_poll_gap_ns(M, N, K, fused), h->comm_stream);
         if (rc) return rc;
     } else {
         int64_t off = 0;
+        long done = 0;
         uint16_t *c = static_cast<uint16_t *>(C);
         uint16_t *acc = static_cast<uint16_t *>(h->acc);
-        for (int i = 0; i < G; i++) {
-            const int64_t n = cseg_host[i] * tile_elems;
-            rc = fo_wait(cseg_host[i], MM + i, h->comm_stream);  // resets the counter
+        for (int i = 0; i < G;) {
+            const int j = batch_end(cseg_host, G, i, done, wave);
+            long tiles = 0;
+            for (int g = i; g < j; g++) tiles += cseg_host[g];
+            const int64_t n = tiles * tile_elems;
+            rc = j - i == 1 ? fo_wait(cseg_host[i], MM + i, h->comm_stream)  // resets the counter
+                            : fo_wait_groups(j - i, cseg_dev + i, MM + i, h->comm_stream);
             if (rc) return rc;
-            if (acc) {
+            if (acc) {  // the groups of a batch are one contiguous range
                 rc = fo_consumer_reduce(dtype, c + off, acc + off, n, h->comm_stream);
                 if (rc) return rc;
             }
             off += n;
+            done += tiles;
+            i = j;
         }
     }
     return join(h);
@@ -206,6 +232,12 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
     const int64_t seg_stride = (int64_t)M * N / W;
     if (h->acc && h->acc_nelem < (int64_t)M * N) return FO_ERR_ARG;
 
+    const int fused = fused_grid(h, G);
+    int32_t wave = 0;
+    if (!fused) {
+        rc = fo_gemm_wave_tiles(dtype, algo, M, N, &wave);
+        if (rc) return rc;
+    }
     rc = fo_gemm_scatter(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, MM, RA, RE, monitor, algo,
                          h->gemm_stream);
     if (rc) return rc;
@@ -213,32 +245,41 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
     uint16_t *c = static_cast<uint16_t *>(C);
     uint16_t *d = static_cast<uint16_t *>(D);
     uint16_t *acc = static_cast<uint16_t *>(h->acc);
-    const int fused = fused_grid(h, G);
+    // With an accumulator and W > 1 the consumer also writes this rank's chunk of
+    // every group to D (ncclReduceScatter(C+acc -> D+acc/W, n/W) with one rank
+    // present, src/overlap_impl.cu:312-313); otherwise a copy per group does.
+    const bool own_in_consumer = d && acc && W > 1;
     if (fused) {
         rc = fo_wait_reduce_groups(dtype, C, h->acc, MM, cseg_dev, G, tile_elems, W, seg_stride,
-                                   h->workspace, fused, fused_slices((int64_t)M * N, G, fused),
-                                   fused_poll_gap_ns(M, N, K, fused), h->comm_stream);
+                                   own_in_consumer ? D : nullptr, h->rank, h->workspace, fused,
+                                   fused_slices((int64_t)M * N, G, fused), fused_poll_gap_ns(M, N, K, fused),
+                                   h->comm_stream);
         if (rc) return rc;
     }
     int64_t off = 0;
-    for (int i = 0; i < G; i++) {
-        const int64_t n = cseg_host[i] * tile_elems;
+    long done = 0;
+    for (int i = 0; i < G;) {
+        const int j = fused ? i + 1 : batch_end(cseg_host, G, i, done, wave);
         if (!fused) {
-            rc = fo_wait(cseg_host[i], MM + i, h->comm_stream);
+            rc = j - i == 1 ? fo_wait(cseg_host[i], MM + i, h->comm_stream)
+                            : fo_wait_groups(j - i, cseg_dev + i, MM + i, h->comm_stream);
             if (rc) return rc;
-            if (acc) {
-                rc = fo_consumer_reduce_rs(dtype, c + off, acc + off / W, n, W, seg_stride,
-                                           h->comm_stream);
+        }
+        for (int g = i; g < j; g++) {  // each group has its own W chunks: one consumer launch per group
+            const int64_t n = cseg_host[g] * tile_elems;
+            if (!fused && acc) {
+                rc = fo_consumer_reduce_rs_own(dtype, c + off, acc + off / W, n, W, seg_stride,
+                                               own_in_consumer ? d + off / W : nullptr, h->rank, h->comm_stream);
                 if (rc) return rc;
             }
+            if (d && !own_in_consumer)
+                FO_HIP_CHECK(hipMemcpyAsync(d + off / W, c + off + (int64_t)h->rank * (n / W),
+                                            (size_t)(n / W) * 2, hipMemcpyDeviceToDevice,
+                                            h->comm_stream));
+            off += n;
+            done += cseg_host[g];
         }
-        // ncclReduceScatter(C+acc -> D+acc/W, n/W) with one rank present: this
-        // rank's chunk of the group is the sum (src/overlap_impl.cu:312-313).
-        if (d)
-            FO_HIP_CHECK(hipMemcpyAsync(d + off / W, c + off + (int64_t)h->rank * (n / W),
-                                        (size_t)(n / W) * 2, hipMemcpyDeviceToDevice,
-                                        h->comm_stream));
-        off += n;
+        i = j;
     }
     return join(h);
 }

@@ -79,6 +79,14 @@ def wait(expect, MM, index=0, stream=None):
     check(lib().fo_wait(int(expect), _counter_ptr(MM, index), _stream(stream)), "fo_wait")
 
 
+def wait_groups(cseg_dev, MM, first=0, count=None, stream=None):
+    """One launch that waits for groups first..first+count-1 in turn and resets their counters."""
+    count = cseg_dev.numel() - first if count is None else count
+    i32 = 4
+    check(lib().fo_wait_groups(int(count), ctypes.c_void_p(cseg_dev.data_ptr() + first * i32),
+                               _counter_ptr(MM, first), _stream(stream)), "fo_wait_groups")
+
+
 def wait_bounded(expect, MM, index, max_polls, status, stream=None):
     check(lib().fo_wait_bounded(int(expect), _counter_ptr(MM, index), int(max_polls),
                                 _i32(status, "status"), _stream(stream)), "fo_wait_bounded")
@@ -95,11 +103,18 @@ def consumer_reduce_rs(src, acc, W, seg_stride, stream=None):
           "fo_consumer_reduce_rs")
 
 
+def consumer_reduce_rs_own(src, acc, W, seg_stride, own, rank, stream=None):
+    check(lib().fo_consumer_reduce_rs_own(dtype_code(src), _ptr(src, "src"), _ptr(acc, "acc"),
+                                          src.numel(), int(W), int(seg_stride), _ptr(own, "own"), int(rank),
+                                          _stream(stream)), "fo_consumer_reduce_rs_own")
+
+
 def wait_reduce_groups(C, ACC, MM, cseg_dev, tile_elems, workspace, W=1, seg_stride=0, nblocks=0,
-                       slices=0, poll_gap_ns=0, stream=None):
+                       slices=0, poll_gap_ns=0, own=None, rank=0, stream=None):
     check(lib().fo_wait_reduce_groups(dtype_code(C), _ptr(C, "C"), _ptr(ACC, "ACC"), _i32(MM, "MM"),
                                       _i32(cseg_dev, "cSeg"), cseg_dev.numel(), int(tile_elems),
-                                      int(W), int(seg_stride), _i32(workspace, "workspace"),
+                                      int(W), int(seg_stride), _ptr(own, "own"),
+                                      int(rank), _i32(workspace, "workspace"),
                                       int(nblocks), int(slices), int(poll_gap_ns), _stream(stream)), "fo_wait_reduce_groups")
 
 

@@ -60,6 +60,11 @@ int fo_schedule_order(int algo, int M, int N, int32_t *order);
  * One wave of the 256-CU chip completes 256 * tiles_per_workgroup tiles; the
  * reference's tuner uses sm_count - 2 tiles per wave (tune/search.py:404). */
 int fo_workgroup_tiles(int algo, int M, int N, int32_t *tiles_per_workgroup, int32_t *workgroups);
+/* Reorder tiles that complete together: the workgroups the persistent GEMM
+ * keeps resident on the current device times the reorder tiles per workgroup
+ * (needs a GPU: the count comes from the occupancy of the compiled kernel).
+ * The counterpart of sm_count - 2 in tune/search.py:404. */
+int fo_gemm_wave_tiles(int dtype, int algo, int M, int N, int32_t *tiles);
 
 /* ---- GEMM -------------------------------------------------------------
  * C[M,N] = A[M,K] . B[N,K]^T, 16-bit in/out, fp32 accumulate.
@@ -104,6 +109,11 @@ int fo_wait(int expect, int32_t *counter, fo_stream_t stream);
  * success *status is left unchanged.  No counterpart in the reference (its
  * waiter spins forever); exists so that failure handling can be tested
  * without hanging a GPU. */
+/* fo_wait for `count` consecutive groups in one launch: for g = 0..count-1 in
+ * turn, spin until counters[g] == expect_dev[g] (device array, e.g. cSEG_GPU + i),
+ * then reset counters[g].  Used for groups that complete in the same wave of the
+ * GEMM, where one launch per group would only add launch latency. */
+int fo_wait_groups(int count, const int32_t *expect_dev, int32_t *counters, fo_stream_t stream);
 int fo_wait_bounded(int expect, int32_t *counter, int64_t max_polls, int32_t *status,
                     fo_stream_t stream);
 
@@ -119,12 +129,19 @@ int fo_consumer_reduce(int dtype, const void *src, void *acc, int64_t nelem, fo_
  * acc + q*seg_stride (elements).  (nelem/W) % 8 == 0. */
 int fo_consumer_reduce_rs(int dtype, const void *src, void *acc, int64_t nelem, int W,
                           int64_t seg_stride, fo_stream_t stream);
+/* The same, and chunk `rank` of src is also copied to own[0 : nelem/W]: what
+ * ncclReduceScatter(C + acc, D + acc/W, n/W, ...) leaves in D with one rank
+ * present (src/overlap_impl.cu:312-313).  own == NULL: no copy. */
+int fo_consumer_reduce_rs_own(int dtype, const void *src, void *acc, int64_t nelem, int W,
+                              int64_t seg_stride, void *own, int rank, fo_stream_t stream);
 
 /* One launch that does, for every group i in order, what the host loop of
  * src/overlap_impl.cu:250-258 enqueues as 2*G launches: wait until
  * MM[i] == cseg[i], reset MM[i] to 0, then accumulate the group's contiguous
  * range of C into ACC (W == 1) or its W chunks into ACC + q*seg_stride at
  * offset acc/W (W > 1).  ACC == NULL: wait/reset only.  tile_elems = BM*BN.
+ * own != NULL (needs ACC and W > 1): chunk `rank` of every group is also copied
+ * to own + (group offset)/W, the reduce-scatter output with one rank present.
  * The counters are reset by the last workgroup to leave instead of per group.
  * workspace: device int32[2], zero before the first use; the kernel leaves
  * word 0 zero and sets word 1 only if a bounded poll gave up (see
@@ -140,8 +157,8 @@ int fo_consumer_reduce_rs(int dtype, const void *src, void *acc, int64_t nelem, 
  * no acquire fence, so it does not disturb the L2 of a GEMM running beside it. */
 int fo_wait_reduce_groups(int dtype, const void *C, void *ACC, int32_t *MM,
                           const int32_t *cseg_dev, int G, int64_t tile_elems, int W,
-                          int64_t seg_stride, int32_t *workspace, int nblocks, int slices,
-                          int poll_gap_ns, fo_stream_t stream);
+                          int64_t seg_stride, void *own, int rank, int32_t *workspace, int nblocks,
+                          int slices, int poll_gap_ns, fo_stream_t stream);
 
 /* ---- RMSNorm ----------------------------------------------------------
  * Replaces reorder_rmsnorm(X, RX, RW, BM, BN, rldn, RA), src/rmsnorm/rmsnorm.h:6-8,

@@ -156,6 +156,18 @@ def test_wait_bounded_gives_up_and_flags(fo):
     assert status.item() == 0 and MM[0].item() == 0
 
 
+def test_wait_groups_resets_a_run_of_counters(fo):
+    cseg = torch.tensor([3, 5, 7, 9], dtype=torch.int32, device="cuda")
+    MM = torch.tensor([3, 5, 7, 9, 11], dtype=torch.int32, device="cuda")
+    fo.ops.wait_groups(cseg, MM, first=1, count=2)        # groups 1 and 2 only
+    torch.cuda.synchronize()
+    assert MM.tolist() == [3, 0, 0, 9, 11]
+    fo.ops.wait_groups(cseg, MM, first=3)                 # the rest
+    fo.ops.wait_groups(cseg, MM, first=0, count=1)
+    torch.cuda.synchronize()
+    assert MM.tolist() == [0, 0, 0, 0, 11]
+
+
 def test_wait_released_by_second_stream(fo):
     MM = torch.zeros(4, dtype=torch.int32, device="cuda")
     status = torch.zeros(1, dtype=torch.int32, device="cuda")
