@@ -79,7 +79,19 @@ def main():
     algo = fo._capi.find_algo(BM, BN, swizzle=args.swizzle)
     TM, TN = M // BM, N // BN
     T = TM * TN
-    cseg = fo.layout.cseg_from_waves(T, gtiles)
+    if args.workload == "c3" and not args.group_tiles:
+        # wave-group sizes chosen by the predictive search (tune/search.py:442-502) from a measured
+        # GEMM duration and the consumer's measured bandwidth curve
+        from flashoverlap_amd import tune
+        Ap = torch.randn(M, K, device="cuda").to(td)
+        Bp = torch.randn(N, K, device="cuda").to(td)
+        Cpp = torch.empty(M, N, device="cuda", dtype=td)
+        dur = tune._time_ms(lambda: ops.gemm(Ap, Bp, Cpp, algo), 10, 20)
+        curve = tune.consumer_bandwidth_curve(td, points=36, warmup=2, reps=5).numpy()
+        cseg, _ = tune.predictive_search(M, N, dur, curve, T, fo._capi.wave_tiles(algo, M, N))
+        del Ap, Bp, Cpp
+    else:
+        cseg = fo.layout.cseg_from_waves(T, gtiles)
     hint = fo._capi.schedule_order(algo, M, N)
     RA = fo.layout.reorder_indices(T, hint, device="cuda").reshape(TM, TN)
     RE = fo.layout.generate_row_mapping(M, N, BM, BN, cseg, W, device="cuda") if W else None
@@ -89,7 +101,11 @@ def main():
         A16 = ((torch.rand(M, K, generator=g) * 2 - 1) * K ** -0.5).to(td)
         B16 = ((torch.rand(N, K, generator=g) * 2 - 1) * K ** -0.5).to(td)
     else:
-        A16 = torch.randn(M, K, generator=g).to(td)
+        A32 = torch.randn(M, K, generator=g)
+        if args.workload == "c3":  # 5 % outlier columns scaled x8
+            cols = torch.randperm(K, generator=g)[: (K * 5 + 99) // 100]
+            A32[:, cols] *= 8
+        A16 = A32.to(td)
         B16 = (torch.randn(N, K, generator=g) * K ** -0.5).to(td)
     gamma16 = (1 + 0.01 * torch.randn(N, generator=g)).to(td)
     A, B, gamma = A16.cuda(), B16.cuda(), gamma16.cuda()
@@ -213,7 +229,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dt, "data": "synthetic",
         "config": {"workload": f"{args.workload}: {desc}", "M": M, "N": N, "K": K, "tile": [BM, BN],
-                   "groups": len(cseg), "algo": algo,
+                   "groups": len(cseg), "cseg": cseg if len(cseg) <= 16 else f"{len(cseg)} x {cseg[0]}", "algo": algo,
                    "consumer_launches": "per-group" if (args.fused == 0 or (args.fused < 0 and len(cseg) <= 16))
                    else "one"},
         "roofline": {"bound": "mfma", "kernel": "fo_gemm_kernel (signal epilogue)",

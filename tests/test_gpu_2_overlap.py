@@ -344,3 +344,18 @@ def test_predictive_search_on_measured_curve(fo):
     assert wave == 512                                # 256 CUs x two 256x128 tiles per 256x256 workgroup
     cseg, est = tune.predictive_search(M, N, 0.4, curve, 2048, wave)
     assert sum(cseg) == 2048 and est > 0.4
+
+
+def test_speed_table_from_a_tuned_config(fo, tmp_path, capsys):
+    """Tune a small shape, then print the reference's speed table for it (test/test.py:325-372)."""
+    from flashoverlap_amd import tune, speed
+    M, N, K = 4096, 4096, 128
+    tune.tune_shape(M, N, K, directory=str(tmp_path), candidates=2, reps=6, quiet=True)
+    speed.WARM_UP, speed.REP = 3, 10
+    speed.main(["--m", str(M), "--n", str(N), "--k", str(K), "--path", str(tmp_path)])
+    out = capsys.readouterr().out
+    for key in ("tile_num", "gemm_dur (ms)", "comm_dur (ms)", "baseline_dur (ms)", "overlap_dur (ms)", "speedup"):
+        assert key in out
+    data = fo.config.load_solution(M, N, K, directory=str(tmp_path))
+    comm, over, base = speed.measure(M, N, K, data, "reduce_scatter", world=8, warmup=2, reps=5)
+    assert comm > 0 and over > 0 and base > 0
