@@ -33,6 +33,7 @@ SIGNATURES = {
     "fo_consumer_reduce": (c_int, [c_int, vp, vp, c_i64, vp]),
     "fo_consumer_reduce_rs": (c_int, [c_int, vp, vp, c_i64, c_int, c_i64, vp]),
     "fo_consumer_reduce_rs_own": (c_int, [c_int, vp, vp, c_i64, c_int, c_i64, vp, c_int, vp]),
+    "fo_consumer_reduce_rs_groups": (c_int, [c_int, vp, vp, vp, c_int, c_i64, c_i64, c_int, c_i64, vp, c_int, vp]),
     "fo_wait_reduce_groups": (c_int, [c_int, vp, vp, vp, vp, c_int, c_i64, c_int, c_i64, vp, c_int, vp,
                                       c_int, c_int, c_int, vp]),
     "fo_reorder_rmsnorm": (c_int, [c_int, vp, vp, vp, c_int, c_int, c_int, c_int, c_int, vp, c_f32,

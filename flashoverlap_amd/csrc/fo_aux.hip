@@ -150,6 +150,26 @@ __global__ __launch_bounds__(CONSUMER_THREADS, 8) void fo_consumer_kernel(const 
                                        rank);
 }
 
+// The same for `ngroups` consecutive groups in one launch (blockIdx.y = group):
+// group k holds cseg[k] tiles of tile16 16-byte units and starts where group
+// k-1 ends; each group is cut into its own W chunks.  src, acc and own point at
+// the first group's range (acc and own at offset/W of it).
+template <typename Tag>
+__global__ __launch_bounds__(CONSUMER_THREADS, 8) void fo_consumer_groups_kernel(
+    const fo_u32x4 *src, fo_u32x4 *acc, const int32_t *cseg, long tile16, int W, long seg_stride16,
+    fo_u32x4 *own, int rank) {
+    long off = 0;
+    for (int k = 0; k < (int)blockIdx.y; k++) off += cseg[k];
+    off *= tile16;
+    const long total = (long)cseg[blockIdx.y] * tile16;
+    const long per = (total + gridDim.x - 1) / gridDim.x;
+    const long lo = per * blockIdx.x;
+    const long hi = lo + per < total ? lo + per : total;
+    if (lo >= hi) return;
+    reduce_range<Tag, true, false>(src + off, acc + off / W, lo, hi, total / W, seg_stride16, threadIdx.x,
+                                   blockDim.x, own ? own + off / W : nullptr, rank);
+}
+
 // One launch for all groups.  The work is cut into items (group g, slice s of
 // that group's contiguous range); workgroup b owns items b, b+nb, b+2nb, ...
 // in ascending order.  With as many slices as workgroups every workgroup takes
@@ -384,6 +404,32 @@ extern "C" int fo_consumer_reduce_rs_own(int dtype, const void *src, void *acc, 
     else if (dtype == FO_BF16)
         hipLaunchKernelGGL(fo_consumer_kernel<fo_bf16_tag>, grid, block, 0, s, (const fo_u32x4 *)src,
                            (fo_u32x4 *)acc, chunk16, W, (long)(seg_stride / 8), (fo_u32x4 *)own, rank);
+    else
+        return FO_ERR_DTYPE;
+    FO_LAUNCH_CHECK();
+    return FO_OK;
+}
+
+extern "C" int fo_consumer_reduce_rs_groups(int dtype, const void *src, void *acc, const int32_t *cseg_dev,
+                                            int ngroups, int64_t max_group_tiles, int64_t tile_elems, int W,
+                                            int64_t seg_stride, void *own, int rank, fo_stream_t stream) {
+    if (!src || !acc || !cseg_dev || ngroups <= 0 || max_group_tiles <= 0 || tile_elems <= 0 || W < 2)
+        return FO_ERR_ARG;
+    if (own && (rank < 0 || rank >= W)) return FO_ERR_ARG;
+    if (tile_elems % (8 * W) || seg_stride % 8) return FO_ERR_SHAPE;
+    if (((uintptr_t)src | (uintptr_t)acc | (uintptr_t)own) & 15) return FO_ERR_SHAPE;
+    const long tile16 = tile_elems / 8;
+    int per_group = consumer_grid(max_group_tiles * tile16);
+    if ((long)per_group * ngroups > 2 * CONSUMER_MAX_BLOCKS) per_group = 2 * CONSUMER_MAX_BLOCKS / ngroups;
+    if (per_group < 1) per_group = 1;
+    dim3 grid(per_group, ngroups), block(CONSUMER_THREADS);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == FO_F16)
+        hipLaunchKernelGGL(fo_consumer_groups_kernel<fo_f16_tag>, grid, block, 0, s, (const fo_u32x4 *)src,
+                           (fo_u32x4 *)acc, cseg_dev, tile16, W, (long)(seg_stride / 8), (fo_u32x4 *)own, rank);
+    else if (dtype == FO_BF16)
+        hipLaunchKernelGGL(fo_consumer_groups_kernel<fo_bf16_tag>, grid, block, 0, s, (const fo_u32x4 *)src,
+                           (fo_u32x4 *)acc, cseg_dev, tile16, W, (long)(seg_stride / 8), (fo_u32x4 *)own, rank);
     else
         return FO_ERR_DTYPE;
     FO_LAUNCH_CHECK();

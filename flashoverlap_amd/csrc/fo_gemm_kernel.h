@@ -452,6 +452,15 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
                                                  : (long)(r % p.rLDN) * p.BN + col0;
             char *cbase = reinterpret_cast<char *>(p.C) + (trow * ldp + tcol) * 2;  // wave-uniform
             const unsigned lane_off = (unsigned)(srow * ldp + scol * 8) * 2;
+            // scatter: the row map entries of all rows this lane will store, fetched in one batch
+            int32_t dest_row[MODE == MODE_SCATTER ? FM * (32 / RPP) : 1];
+            if (MODE == MODE_SCATTER) {
+#pragma unroll
+                for (int i = 0; i < FM; i++)
+#pragma unroll
+                    for (int ps = 0; ps < 32 / RPP; ps++)
+                        dest_row[i * (32 / RPP) + ps] = p.RE[trow + i * 32 + ps * RPP + srow];
+            }
 #pragma unroll
             for (int i = 0; i < FM; i++) {
 #pragma unroll
@@ -478,7 +487,7 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
                     fo_u32x4 v = *reinterpret_cast<const fo_u32x4 *>(strip + row * PITCH + scol * 8);
                     if (MODE == MODE_SCATTER) {
                         // rows go through the row map: per-lane 64-bit address
-                        const long prow = p.RE[trow + i * 32 + row];
+                        const long prow = dest_row[i * (32 / RPP) + ps];
                         store16_write_through(p.C + (size_t)prow * ldp + tcol + scol * 8, v);
                     } else {
                         char *sb = cbase + (size_t)(i * 32 + ps * RPP) * ldp * 2;

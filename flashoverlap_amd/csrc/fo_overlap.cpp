@@ -265,9 +265,18 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
                             : fo_wait_groups(j - i, cseg_dev + i, MM + i, h->comm_stream);
             if (rc) return rc;
         }
-        for (int g = i; g < j; g++) {  // each group has its own W chunks: one consumer launch per group
+        if (!fused && acc && W > 1 && j - i > 1) {
+            // the groups of one wave in one launch; each keeps its own W chunks
+            long most = 0;
+            for (int g = i; g < j; g++) most = cseg_host[g] > most ? cseg_host[g] : most;
+            rc = fo_consumer_reduce_rs_groups(dtype, c + off, acc + off / W, cseg_dev + i, j - i, most, tile_elems,
+                                              W, seg_stride, own_in_consumer ? d + off / W : nullptr, h->rank,
+                                              h->comm_stream);
+            if (rc) return rc;
+        }
+        for (int g = i; g < j; g++) {
             const int64_t n = cseg_host[g] * tile_elems;
-            if (!fused && acc) {
+            if (!fused && acc && !(W > 1 && j - i > 1)) {
                 rc = fo_consumer_reduce_rs_own(dtype, c + off, acc + off / W, n, W, seg_stride,
                                                own_in_consumer ? d + off / W : nullptr, h->rank, h->comm_stream);
                 if (rc) return rc;

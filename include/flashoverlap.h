@@ -134,6 +134,13 @@ int fo_consumer_reduce_rs(int dtype, const void *src, void *acc, int64_t nelem, 
  * present (src/overlap_impl.cu:312-313).  own == NULL: no copy. */
 int fo_consumer_reduce_rs_own(int dtype, const void *src, void *acc, int64_t nelem, int W,
                               int64_t seg_stride, void *own, int rank, fo_stream_t stream);
+/* The same for ngroups consecutive groups in one launch (W >= 2): group k has
+ * cseg_dev[k] tiles of tile_elems elements and its own W chunks; src, acc and own
+ * point at the first group's range (acc and own at offset/W).  max_group_tiles
+ * (the largest cseg of the run, known on the host) sizes the grid. */
+int fo_consumer_reduce_rs_groups(int dtype, const void *src, void *acc, const int32_t *cseg_dev,
+                                 int ngroups, int64_t max_group_tiles, int64_t tile_elems, int W,
+                                 int64_t seg_stride, void *own, int rank, fo_stream_t stream);
 
 /* One launch that does, for every group i in order, what the host loop of
  * src/overlap_impl.cu:250-258 enqueues as 2*G launches: wait until
