@@ -261,6 +261,7 @@ __global__ __launch_bounds__(256) void fo_rmsnorm_kernel(const fo_u32x4 *X, fo_u
     const int ldn = RA ? dim / BN : 0;
     const int tile_row = RA ? b / BM : 0, in_row = RA ? b % BM : 0;
     const long ldp16 = RA ? ((long)rldn * BN) >> 3 : 0;
+    const int bn_shift = (RA && rldn == 1 && (BN & (BN - 1)) == 0) ? __builtin_ctz(BN) : -1;
 
     fo_u32x4 x[MAXCH];
     float ss = 0.f;
@@ -271,10 +272,17 @@ __global__ __launch_bounds__(256) void fo_rmsnorm_kernel(const fo_u32x4 *X, fo_u
             long src;
             if (RA) {
                 const int j = c << 3;
-                const int r = RA[tile_row * ldn + j / BN];
-                const long nr = (long)(r / rldn) * BM + in_row;
-                const int nc = (r % rldn) * BN + j % BN;
-                src = nr * ldp16 + (nc >> 3);
+                if (bn_shift >= 0) {
+                    // rldn == 1 and BN a power of two (every tile of the Algo table): tile r is
+                    // the contiguous block of BM rows of BN columns that starts at row r * BM
+                    const int r = RA[tile_row * ldn + (j >> bn_shift)];
+                    src = ((long)r * BM + in_row) * ldp16 + ((j & (BN - 1)) >> 3);
+                } else {
+                    const int r = RA[tile_row * ldn + j / BN];
+                    const long nr = (long)(r / rldn) * BM + in_row;
+                    const int nc = (r % rldn) * BN + j % BN;
+                    src = nr * ldp16 + (nc >> 3);
+                }
             } else {
                 src = (long)b * nch + c;
             }
@@ -350,6 +358,9 @@ long default_max_polls() {
 }
 
 int consumer_grid(long n16) {
+    // Ranges far beyond the last-level cache stream best from 128 workgroups, each on one
+    // long contiguous piece (measured on 8192^2: 7.0 TB/s against 6.7 TB/s for 256 or more).
+    if (n16 >= (4L << 20)) return 128;
     long blocks = (n16 + CONSUMER_THREADS * CONSUMER_UNROLL - 1) / (CONSUMER_THREADS * CONSUMER_UNROLL);
     if (blocks < 1) blocks = 1;
     if (blocks > 2 * CONSUMER_MAX_BLOCKS) blocks = 2 * CONSUMER_MAX_BLOCKS;  // it does not spin: two per CU are fine

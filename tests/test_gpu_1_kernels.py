@@ -251,7 +251,7 @@ def test_rmsnorm_constant_row_closed_form(fo):
 @pytest.mark.parametrize("dtype", [F16, BF16])
 def test_reorder_rmsnorm_undoes_the_permutation(fo, oracle, dtype):
     for (bm, bn, M, N, rldn) in [(128, 128, 256, 1024, 1), (128, 256, 256, 4096, 1), (64, 128, 256, 512, 2),
-                                 (16, 128, 64, 8192, 1)]:
+                                 (16, 128, 64, 8192, 1), (32, 96, 64, 480, 1)]:  # last: BN no power of two
         TM, TN = M // bm, N // bn
         T = TM * TN
         rng = np.random.default_rng(40)
