@@ -359,3 +359,36 @@ def test_speed_table_from_a_tuned_config(fo, tmp_path, capsys):
     data = fo.config.load_solution(M, N, K, directory=str(tmp_path))
     comm, over, base = speed.measure(M, N, K, data, "reduce_scatter", world=8, warmup=2, reps=5)
     assert comm > 0 and over > 0 and base > 0
+
+
+@pytest.mark.parametrize("fused", [0, 1])
+def test_consumer_never_reads_a_stale_tile(fo, fused):
+    """Back-to-back overlapped calls on the same buffers with different operands: every
+    group the consumer adds must be the tile values of the current call, never what a
+    cache still holds from the previous one (the tiles are written through on one XCD
+    and read, moments after the signal, on others)."""
+    M, N, K, bm, bn = 4096, 4096, 256, 128, 128
+    cseg = [128] * 8
+    algo, RA, A1, B, _, _, MM, cs_cpu, cs_gpu = _setup(fo, F16, bm, bn, M, N, K, cseg, swizzle=4, seed=80)
+    ops = fo.ops
+    Cp = torch.empty(M * N, device="cuda", dtype=torch.float16)
+    ACC = torch.zeros(M * N, device="cuda", dtype=torch.float16)
+    Y = torch.empty(M, N, device="cuda", dtype=torch.float16)
+    gamma = torch.ones(N, device="cuda", dtype=torch.float16)
+    ov = ops.Overlap()
+    ov.set_accumulator(ACC)
+    ov.set_fused_consumer(fused)
+    expect = torch.zeros(M * N, device="cuda", dtype=torch.float32)
+    ref = torch.empty(M * N, device="cuda", dtype=torch.float16)
+    mm_ref = torch.zeros_like(MM)
+    for it in range(6):
+        A = (A1 * (0.25 * (it + 1))).roll(it * 37, dims=0).contiguous()   # a different product every call
+        ov.gemm_allreduce_overlap(A, B, Cp, MM, RA, 1, cs_cpu, cs_gpu, algo)
+        ops.reorder_rmsnorm(Cp.view(M, N), Y, gamma, bm, bn, 1, RA, eps=1e-6)   # reads all of Cp into the caches
+        ops.gemm_signal(A, B, ref, mm_ref, RA, cs_gpu, algo)
+        mm_ref.zero_()
+        expect = (expect + ref.float()).half().float()
+    torch.cuda.synchronize()
+    assert torch.equal(ACC.float(), expect)
+    assert (MM == 0).all()
+    ov.close()
