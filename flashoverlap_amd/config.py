@@ -15,14 +15,15 @@ DEFAULT_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__fil
 
 def gpu_tag(device_name=None):
     """The reference slices characters 7..10 of the device name ("NVIDIA A800..." -> "a800");
-    "AMD Instinct MI355X" gives "tinc".  FLASHOVERLAP_GPU_TAG overrides."""
+    "AMD Instinct MI355X" gives "tinc".  Blanks are trimmed (a name like "AMD Radeon Graphics"
+    would otherwise put a space into the file name).  FLASHOVERLAP_GPU_TAG overrides."""
     tag = os.environ.get("FLASHOVERLAP_GPU_TAG")
     if tag:
         return tag
     if device_name is None:
         import torch
         device_name = torch.cuda.get_device_properties(torch.cuda.current_device()).name
-    return device_name[7:11].lower()
+    return device_name[7:11].lower().strip().replace(" ", "_")
 
 
 def config_path(M, N, K, gpu=None, directory=None):

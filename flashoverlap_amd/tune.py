@@ -97,7 +97,17 @@ def predictive_search(M, N, gemm_dur, curve, tile_num, wave, full_wave=None,
 
 
 # ------------------------------------------------------------------ measurement (GPU)
-def _time_ms(fn, warmup, reps):
+def _time_ms(fn, warmup, reps, settle_s=0.0):
+    """Mean ms per call from per-call device events.  settle_s > 0 first keeps the GPU busy with
+    fn for that long: for the first few dozen launches after an idle gap (allocations, host work)
+    the part runs up to 30 % slower, which would otherwise decide between candidates."""
+    if settle_s > 0:
+        import time
+        t_end = time.perf_counter() + settle_s
+        while time.perf_counter() < t_end:
+            for _ in range(10):
+                fn()
+            torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     start = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
@@ -117,10 +127,12 @@ def profile_gemm_configs(M, N, K, dtype=torch.float16, top=10, warmup=10, reps=1
     B = torch.randn(N, K, device="cuda").to(dtype)
     C = torch.empty(M, N, device="cuda", dtype=dtype)
     rows = []
+    settle = 0.3  # before the first candidate only: the candidates follow each other without a gap
     for algo, row in enumerate(_capi.algo_table()):
         if M % row[0] or N % row[1]:
             continue
-        rows.append((_time_ms(lambda: ops.gemm(A, B, C, algo), warmup, reps), row[0], row[1], algo))
+        rows.append((_time_ms(lambda: ops.gemm(A, B, C, algo), warmup, reps, settle), row[0], row[1], algo))
+        settle = 0.0
     rows.sort()
     rows = rows[:top]
     return [r[1] for r in rows], [r[2] for r in rows], [r[0] for r in rows], [r[3] for r in rows]
@@ -197,10 +209,10 @@ def time_overlap(M, N, K, algo, cseg, hint, dtype=torch.float16, warmup=20, reps
     if with_consumer:
         ov.set_accumulator(torch.zeros(M * N, device="cuda", dtype=dtype))
     if len(cseg) == 1:
-        ms = _time_ms(lambda: ov.gemm_allreduce(A, B, C, algo), warmup, reps)
+        ms = _time_ms(lambda: ov.gemm_allreduce(A, B, C, algo), warmup, reps, settle_s=0.2)
     else:
         ms = _time_ms(lambda: ov.gemm_allreduce_overlap(A, B, C, MM, RA, 1, cseg_cpu, cseg_gpu, algo),
-                      warmup, reps)
+                      warmup, reps, settle_s=0.2)
     torch.cuda.synchronize()
     ov.close()
     return ms
