@@ -249,8 +249,10 @@ __global__ __launch_bounds__(CONSUMER_THREADS, 8) void fo_wait_reduce_kernel(
 // 16-byte chunks of the row in registers between the sum of squares and the
 // scaling, so the row is read once.  With RA != nullptr the chunks are gathered
 // from the tile-reordered buffer (index math of src/rmsnorm/rmsnorm.cuh:80-86).
+// The second launch bound caps the registers (128 up to 16 chunks per lane, 256 above) so that
+// enough wavefronts stay resident to cover the memory latency.
 template <typename Tag, int MAXCH>
-__global__ __launch_bounds__(256) void fo_rmsnorm_kernel(const fo_u32x4 *X, fo_u32x4 *Y, const fo_u32x4 *Wt,
+__global__ __launch_bounds__(256, MAXCH <= 16 ? 4 : 2) void fo_rmsnorm_kernel(const fo_u32x4 *X, fo_u32x4 *Y, const fo_u32x4 *Wt,
                                                          int bs, int dim, int BM, int BN, int rldn,
                                                          const int32_t *RA, float eps) {
     typedef fo_elem<Tag> E;

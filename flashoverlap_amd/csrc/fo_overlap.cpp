@@ -9,6 +9,7 @@ struct fo_overlap {
     hipStream_t gemm_stream = nullptr;
     hipStream_t comm_stream = nullptr;
     hipEvent_t joined = nullptr;
+    hipEvent_t forked = nullptr;
     int32_t *workspace = nullptr;  // zeroed words of the one-launch wait+reduce kernel
     bool gemm_ready = false;
     bool overlap_ready = false;
@@ -77,6 +78,17 @@ int check_segments(const int32_t *cseg_host, int G, long tiles) {
     return sum == tiles ? FO_OK : FO_ERR_SEGMENTS;
 }
 
+// GEMM stream -> consumer stream, recorded right before the GEMM is enqueued.  Only the
+// one-launch consumer needs it: its workgroups poll from the moment they start, and polls
+// slow down whatever shares the memory system with them, so they must not start while the
+// GEMM stream is still busy with the work that precedes the GEMM (the reference's wait
+// kernels may start early: a single sleeping lane disturbs nobody).
+int fork(fo_overlap *h) {
+    FO_HIP_CHECK(hipEventRecord(h->forked, h->gemm_stream));
+    FO_HIP_CHECK(hipStreamWaitEvent(h->comm_stream, h->forked, 0));
+    return FO_OK;
+}
+
 // consumer stream -> GEMM stream, as the event pair at src/overlap_impl.cu:260-263.
 int join(fo_overlap *h) {
     FO_HIP_CHECK(hipEventRecord(h->joined, h->comm_stream));
@@ -99,6 +111,7 @@ extern "C" int fo_overlap_destroy(fo_overlap_t *h) {
         hipStreamDestroy(h->comm_stream);
     }
     if (h->joined) hipEventDestroy(h->joined);
+    if (h->forked) hipEventDestroy(h->forked);
     if (h->workspace) hipFree(h->workspace);
     delete h;
     return FO_OK;
@@ -118,6 +131,7 @@ extern "C" int fo_overlap_init(fo_overlap_t *h) {
     // src/overlap_impl.cu:140): mixed-priority streams are avoided on this platform.
     FO_HIP_CHECK(hipStreamCreateWithFlags(&h->comm_stream, hipStreamNonBlocking));
     FO_HIP_CHECK(hipEventCreateWithFlags(&h->joined, hipEventDisableTiming));
+    FO_HIP_CHECK(hipEventCreateWithFlags(&h->forked, hipEventDisableTiming));
     FO_HIP_CHECK(hipMalloc(&h->workspace, 64));
     FO_HIP_CHECK(hipMemset(h->workspace, 0, 64));
     h->overlap_ready = true;
@@ -178,6 +192,10 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
         rc = fo_gemm_wave_tiles(dtype, algo, M, N, &wave);
         if (rc) return rc;
     }
+    if (fused) {
+        rc = fork(h);
+        if (rc) return rc;
+    }
     rc = fo_gemm_signal(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, MM, RA, monitor, algo,
                         h->gemm_stream);
     if (rc) return rc;  // nothing has been enqueued on the consumer stream yet
@@ -236,6 +254,10 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
     int32_t wave = 0;
     if (!fused) {
         rc = fo_gemm_wave_tiles(dtype, algo, M, N, &wave);
+        if (rc) return rc;
+    }
+    if (fused) {
+        rc = fork(h);
         if (rc) return rc;
     }
     rc = fo_gemm_scatter(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, MM, RA, RE, monitor, algo,
