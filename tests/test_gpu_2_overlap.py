@@ -392,3 +392,32 @@ def test_consumer_never_reads_a_stale_tile(fo, fused):
     assert torch.equal(ACC.float(), expect)
     assert (MM == 0).all()
     ov.close()
+
+
+def test_uneven_tile_walk_matches_vendor_gemm(fo):
+    """1089 workgroup tiles on 256 resident workgroups (65 of them walk five tiles, the rest four),
+    a tile count that is no multiple of 8 (no XCD de-interleave): plain GEMM against torch's GEMM,
+    signal GEMM against the plain one through the inverse permutation, counters exact."""
+    M = N = 8448
+    K = 512
+    bm, bn = 128, 256
+    algo = fo._capi.find_algo(bm, bn, swizzle=4)
+    TM, TN = M // bm, N // bn
+    T = TM * TN
+    g = torch.Generator(device="cuda").manual_seed(5)
+    A = torch.randn(M, K, device="cuda", generator=g).half()
+    B = (torch.randn(N, K, device="cuda", generator=g) * K ** -0.5).half()
+    C = torch.empty(M, N, device="cuda", dtype=torch.float16)
+    fo.ops.gemm(A, B, C, algo)
+    ref = A.float() @ B.float().t()
+    err = (C.float() - ref).abs().max().item() / ref.abs().max().item()
+    assert err <= 2e-3
+    assert max_rel_err(C[::97, ::89].float().cpu(), ref[::97, ::89].cpu()) <= REL_TOL
+    cseg = fo.layout.cseg_from_waves(T, 300)
+    RA = fo.layout.reorder_indices(T, fo._capi.schedule_order(algo, M, N), device="cuda").reshape(TM, TN)
+    MM = torch.zeros(fo.layout.counter_size(len(cseg), TM, TN), dtype=torch.int32, device="cuda")
+    Cp = torch.empty(M * N, device="cuda", dtype=torch.float16)
+    fo.ops.gemm_signal(A, B, Cp, MM, RA, torch.tensor(cseg, dtype=torch.int32, device="cuda"), algo)
+    torch.cuda.synchronize()
+    assert MM[:len(cseg)].tolist() == cseg
+    assert torch.equal(fo.layout.unpermute(Cp, M, N, bm, bn, RA), C)
