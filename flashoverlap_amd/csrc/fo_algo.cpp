@@ -58,7 +58,7 @@ int fo_pick_raster(int algo, int M, int N, fo_raster *r) {
     r->grid_m = M / r->mtm;
     r->grid_n = N / r->mtn;
     r->panel = e->f[10] < r->grid_m ? e->f[10] : r->grid_m;
-    r->xcd_remap = ((r->grid_m * r->grid_n) % 8 == 0) ? 1 : 0;
+    r->xcd_remap = (r->grid_m * r->grid_n >= 16) ? 1 : 0;
     return FO_OK;
 }
 

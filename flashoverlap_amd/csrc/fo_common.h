@@ -82,9 +82,12 @@ __host__ __device__ inline void fo_wg_to_tile(int wg, int grid_m, int grid_n, in
     int nt = grid_m * grid_n;
     int v = wg;
     if (xcd_remap) {
-        // Workgroups are dealt round-robin to the 8 XCDs; give each XCD one
-        // contiguous range of the raster so its private L2 sees neighbouring tiles.
-        v = (wg & 7) * (nt >> 3) + (wg >> 3);
+        // Workgroups (and, in the persistent walk, tile slots) are dealt round-robin to the
+        // 8 XCDs; give each XCD one contiguous range of the raster so that its private L2
+        // sees neighbouring tiles.  XCD x owns the slots x, x+8, ...: nt/8 of them, one more
+        // for the first nt%8 XCDs.
+        const int q = nt >> 3, rem = nt & 7, x = wg & 7;
+        v = x * q + (x < rem ? x : rem) + (wg >> 3);
     }
     int per_panel = panel * grid_n;
     int p = v / per_panel;
