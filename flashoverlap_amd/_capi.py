@@ -39,6 +39,7 @@ SIGNATURES = {
     "fo_reorder_rmsnorm": (c_int, [c_int, vp, vp, vp, c_int, c_int, c_int, c_int, c_int, vp, c_f32,
                                    vp]),
     "fo_rmsnorm": (c_int, [c_int, vp, vp, vp, c_int, c_int, c_f32, vp]),
+    "fo_overlap_plan_batches": (c_int, [vp, c_int, c_int, vp]),
     "fo_overlap_create": (c_int, [ctypes.POINTER(vp)]),
     "fo_overlap_destroy": (c_int, [vp]),
     "fo_overlap_set_gemm_stream": (c_int, [vp, vp]),
@@ -129,3 +130,14 @@ def wave_tiles(algo, M, N, dtype=F16):
     tiles = ctypes.c_int32()
     check(lib().fo_gemm_wave_tiles(int(dtype), int(algo), M, N, ctypes.byref(tiles)), "fo_gemm_wave_tiles")
     return tiles.value
+
+
+def plan_batches(cseg, wave_tiles):
+    """Groups per launch of the per-group consumer path: list of (first_group, end_group)."""
+    G = len(cseg)
+    arr = (ctypes.c_int32 * G)(*cseg)
+    first = (ctypes.c_int32 * (G + 1))()
+    n = lib().fo_overlap_plan_batches(arr, G, int(wave_tiles), first)
+    if n < 0:
+        raise FlashOverlapError("fo_overlap_plan_batches", n)
+    return [(first[i], first[i + 1]) for i in range(n)]

@@ -98,6 +98,22 @@ int join(fo_overlap *h) {
 
 }  // namespace
 
+extern "C" int fo_overlap_plan_batches(const int32_t *cseg_host, int G, int wave_tiles, int32_t *first) {
+    if (!cseg_host || !first || G <= 0) return FO_ERR_ARG;
+    for (int i = 0; i < G; i++)
+        if (cseg_host[i] <= 0) return FO_ERR_SEGMENTS;
+    int n = 0;
+    long done = 0;
+    for (int i = 0; i < G;) {
+        const int j = batch_end(cseg_host, G, i, done, wave_tiles);
+        first[n++] = i;
+        for (int g = i; g < j; g++) done += cseg_host[g];
+        i = j;
+    }
+    first[n] = G;
+    return n;
+}
+
 extern "C" int fo_overlap_create(fo_overlap_t **out) {
     if (!out) return FO_ERR_ARG;
     *out = new (std::nothrow) fo_overlap();

@@ -200,6 +200,13 @@ int fo_overlap_set_world(fo_overlap_t *h, int rank, int world);
  * reduces across ranks in place).  acc == NULL detaches it.  For W > 1 it is
  * [W, M/W, N] (seg_stride = M/W*N elements). */
 int fo_overlap_set_accumulator(fo_overlap_t *h, void *acc, int64_t nelem);
+/* How the per-group consumer path batches its launches (host-only, no GPU
+ * needed): groups whose last tiles fall into the same stretch of wave_tiles
+ * consecutive storage slots complete together and share one wait and one
+ * consumer launch.  first[0..n] receives the first group of each batch and G
+ * at the end (room for G + 1 entries); returns n, or a negative error.
+ * wave_tiles <= 0: no batching. */
+int fo_overlap_plan_batches(const int32_t *cseg_host, int G, int wave_tiles, int32_t *first);
 /* fused < 0 (default): chosen per call, one launch when there are more than 16
  * groups; 0: always 2*G launches as the reference's host loop
  * (src/overlap_impl.cu:250-258); 1: always one fo_wait_reduce_groups launch

@@ -157,3 +157,20 @@ def test_layout_matches_checker_on_random_cases(oracle):
         got = layout.generate_row_mapping(TM * BM, TN * BN, BM, BN, cseg, W, device="cpu")
         assert got.tolist() == oracle.row_mapping(TM * BM, TN * BN, BM, BN, cseg, W).tolist()
         assert layout.tile_groups(cseg).tolist() == [oracle.tile_group(cseg, r) for r in range(T)]
+
+
+def test_same_wave_groups_share_a_launch():
+    plan = _capi.plan_batches
+    # large square: 8 groups of 256 tiles, 512 tiles complete per wave -> pairs
+    assert plan([256] * 8, 512) == [(0, 2), (2, 4), (4, 6), (6, 8)]
+    # reduce-scatter layout: 1024 tiles per wave -> four groups per launch
+    assert plan([256] * 8, 1024) == [(0, 4), (4, 8)]
+    # a group that straddles a wave boundary completes with the later wave
+    assert plan([300, 300, 300, 124], 512) == [(0, 1), (1, 2), (2, 4)]
+    # groups of whole waves, and no batching without a wave size
+    assert plan([512, 512, 1024], 512) == [(0, 1), (1, 2), (2, 3)]
+    assert plan([4] * 6, 0) == [(i, i + 1) for i in range(6)]
+    # one wave covers everything
+    assert plan([1, 2, 3], 1000) == [(0, 3)]
+    with pytest.raises(_capi.FlashOverlapError):
+        plan([4, 0, 4], 8)
