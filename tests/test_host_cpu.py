@@ -167,7 +167,7 @@ def test_same_wave_groups_share_a_launch():
     assert plan([256] * 8, 1024) == [(0, 4), (4, 8)]
     # a group that straddles a wave boundary completes with the later wave
     assert plan([300, 300, 300, 124], 512) == [(0, 1), (1, 4)]
-    assert plan([300, 300, 500, 436], 512) == [(0, 1), (1, 2), (2, 3), (3, 4)]
+    assert plan([300, 300, 500, 436], 512) == [(0, 1), (1, 2), (2, 4)]   # ends at 300, 600, 1100, 1536
     # groups of whole waves, and no batching without a wave size
     assert plan([512, 512, 1024], 512) == [(0, 1), (1, 2), (2, 3)]
     assert plan([4] * 6, 0) == [(i, i + 1) for i in range(6)]
