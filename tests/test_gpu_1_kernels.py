@@ -293,3 +293,33 @@ def test_error_codes_on_gpu(fo):
     assert e.value.code == -3
     with pytest.raises(TypeError):
         fo.ops.gemm(A.float(), A.float(), C.float(), 0)
+
+
+def test_reorder_table_changed_in_place_between_launches(fo):
+    """RA and cSeg are read through the scalar cache / an LDS table built at kernel start:
+    a launch must see what the tensors hold at that time, not what an earlier launch read."""
+    bm, bn, M, N, K = 128, 128, 2048, 2048, 128
+    algo = _algo(fo, bm, bn, swizzle=4)
+    TM, TN = M // bm, N // bn
+    T = TM * TN
+    A, _ = seeded((M, K), F16, 31)
+    B, _ = seeded((N, K), F16, 32, scale=K ** -0.5)
+    plain = torch.empty(M, N, device="cuda", dtype=torch.float16)
+    fo.ops.gemm(A, B, plain, algo)
+    RA = torch.empty(TM, TN, dtype=torch.int32, device="cuda")
+    cseg = torch.empty(4, dtype=torch.int32, device="cuda")
+    MM = torch.zeros(fo.layout.counter_size(4, TM, TN), dtype=torch.int32, device="cuda")
+    Cp = torch.empty(M * N, device="cuda", dtype=torch.float16)
+    rng = np.random.default_rng(9)
+    for it in range(4):
+        perm = torch.from_numpy(rng.permutation(T).astype(np.int32)).reshape(TM, TN)
+        cuts = sorted(rng.choice(np.arange(1, T), size=3, replace=False).tolist())
+        groups = [b - a for a, b in zip([0] + cuts, cuts + [T])]
+        RA.copy_(perm)                                   # same device buffers, new contents
+        cseg.copy_(torch.tensor(groups, dtype=torch.int32))
+        Cp.fill_(float("nan"))
+        fo.ops.gemm_signal(A, B, Cp, MM, RA, cseg, algo)
+        torch.cuda.synchronize()
+        assert MM[:4].tolist() == groups
+        assert torch.equal(fo.layout.unpermute(Cp, M, N, bm, bn, RA), plain)
+        MM.zero_()
