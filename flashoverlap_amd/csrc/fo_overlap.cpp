@@ -1,6 +1,6 @@
 // Host orchestration of the overlap path: the counterpart of class OverlapImpl
 // (src/overlap_impl.h:12-43, src/overlap_impl.cu) behind a C handle.  Two HIP
-// streams and one event; every call only enqueues work and returns.
+// streams and two events; every call only enqueues work and returns.
 #include <new>
 
 #include "fo_common.h"
