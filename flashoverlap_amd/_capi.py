@@ -22,6 +22,7 @@ SIGNATURES = {
     "fo_schedule_order": (c_int, [c_int, c_int, c_int, vp]),
     "fo_workgroup_tiles": (c_int, [c_int, c_int, c_int, vp, vp]),
     "fo_gemm_wave_tiles": (c_int, [c_int, c_int, c_int, c_int, vp]),
+    "fo_set": (c_int, [vp, c_int, vp]),
     "fo_wait_groups": (c_int, [c_int, vp, vp, vp]),
     "fo_gemm": (c_int, [c_int, c_int, c_int, c_int, vp, vp, vp, c_int, vp]),
     "fo_gemm_signal": (c_int, [c_int, c_int, c_int, c_int, c_int, vp, c_int, vp, vp, vp, vp, vp,

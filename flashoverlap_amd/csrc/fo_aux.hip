@@ -29,6 +29,11 @@ __global__ void fo_wait_kernel(int expect, int32_t *counter, long max_polls, int
     }
 }
 
+// Sets one word: the other half of a join through memory (see fo_set below).
+__global__ void fo_set_kernel(int32_t *word, int value) {
+    __hip_atomic_store(word, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // The same for `count` consecutive groups, one after the other.
 __global__ void fo_wait_groups_kernel(int count, const int32_t *expect, int32_t *counters, long max_polls) {
     for (int g = 0; g < count; g++) {
@@ -375,6 +380,13 @@ extern "C" int fo_wait(int expect, int32_t *counter, fo_stream_t stream) {
     if (!counter) return FO_ERR_ARG;
     hipLaunchKernelGGL(fo_wait_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream), expect,
                        counter, default_max_polls(), (int32_t *)nullptr);
+    FO_LAUNCH_CHECK();
+    return FO_OK;
+}
+
+extern "C" int fo_set(int32_t *word, int value, fo_stream_t stream) {
+    if (!word) return FO_ERR_ARG;
+    hipLaunchKernelGGL(fo_set_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream), word, value);
     FO_LAUNCH_CHECK();
     return FO_OK;
 }

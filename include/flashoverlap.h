@@ -114,6 +114,11 @@ int fo_wait(int expect, int32_t *counter, fo_stream_t stream);
  * then reset counters[g].  Used for groups that complete in the same wave of the
  * GEMM, where one launch per group would only add launch latency. */
 int fo_wait_groups(int count, const int32_t *expect_dev, int32_t *counters, fo_stream_t stream);
+/* One-lane kernel that stores value into *word.  With fo_wait(value, word, other_stream)
+ * it joins two streams through memory: stream order makes everything enqueued before
+ * fo_set complete (and visible) before the word changes, and the waiting stream continues
+ * a few microseconds later -- an event wait across queues measured about 12 us here. */
+int fo_set(int32_t *word, int value, fo_stream_t stream);
 int fo_wait_bounded(int expect, int32_t *counter, int64_t max_polls, int32_t *status,
                     fo_stream_t stream);
 
