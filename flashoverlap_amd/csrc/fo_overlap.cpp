@@ -1,6 +1,6 @@
 // Host orchestration of the overlap path: the counterpart of class OverlapImpl
 // (src/overlap_impl.h:12-43, src/overlap_impl.cu) behind a C handle.  Two HIP
-// streams and two events; every call only enqueues work and returns.
+// streams and one event; every call only enqueues work and returns.
 #include <new>
 
 #include "fo_common.h"
@@ -8,7 +8,6 @@
 struct fo_overlap {
     hipStream_t gemm_stream = nullptr;
     hipStream_t comm_stream = nullptr;
-    hipEvent_t joined = nullptr;
     hipEvent_t forked = nullptr;
     int32_t *workspace = nullptr;  // zeroed words of the one-launch wait+reduce kernel
     bool gemm_ready = false;
@@ -89,18 +88,14 @@ int fork(fo_overlap *h) {
     return FO_OK;
 }
 
-// consumer stream -> GEMM stream, as the event pair at src/overlap_impl.cu:260-263.
-int join(fo_overlap *h) {
-    FO_HIP_CHECK(hipEventRecord(h->joined, h->comm_stream));
-    FO_HIP_CHECK(hipStreamWaitEvent(h->gemm_stream, h->joined, 0));
-    return FO_OK;
-}
-
-// The same join through memory, used when kernels were the last thing enqueued on the
-// consumer stream: a one-lane kernel there sets workspace word 4, a one-lane wait behind
-// the GEMM on the GEMM's stream consumes it.  The wait cannot start before the GEMM has
-// ended and everything it waits for was enqueued before it.  The GEMM stream continues
-// about 4 us after the consumer's end instead of about 12 us with the event pair.
+// consumer stream -> GEMM stream.  The reference records an event on the consumer stream
+// and makes the GEMM stream wait for it (src/overlap_impl.cu:260-263); an event wait across
+// queues measured about 12 us here, so the join goes through memory instead: a one-lane
+// kernel at the end of the consumer stream sets workspace word 4 (stream order makes all
+// earlier work there complete and visible first), a one-lane wait behind the GEMM on the
+// GEMM's stream consumes it.  The wait cannot start before the GEMM has ended and
+// everything it waits for was enqueued before it; the GEMM stream continues about 4 us
+// after the consumer's end.
 int join_through_memory(fo_overlap *h) {
     int rc = fo_set(h->workspace + 4, 1, h->comm_stream);
     if (rc) return rc;
@@ -137,7 +132,6 @@ extern "C" int fo_overlap_destroy(fo_overlap_t *h) {
         hipStreamSynchronize(h->comm_stream);
         hipStreamDestroy(h->comm_stream);
     }
-    if (h->joined) hipEventDestroy(h->joined);
     if (h->forked) hipEventDestroy(h->forked);
     if (h->workspace) hipFree(h->workspace);
     delete h;
@@ -157,7 +151,6 @@ extern "C" int fo_overlap_init(fo_overlap_t *h) {
     // Default priority on purpose (the reference asks for priority -5,
     // src/overlap_impl.cu:140): mixed-priority streams are avoided on this platform.
     FO_HIP_CHECK(hipStreamCreateWithFlags(&h->comm_stream, hipStreamNonBlocking));
-    FO_HIP_CHECK(hipEventCreateWithFlags(&h->joined, hipEventDisableTiming));
     FO_HIP_CHECK(hipEventCreateWithFlags(&h->forked, hipEventDisableTiming));
     FO_HIP_CHECK(hipMalloc(&h->workspace, 64));
     FO_HIP_CHECK(hipMemset(h->workspace, 0, 64));
@@ -253,9 +246,8 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
             done += tiles;
             i = j;
         }
-        return join_through_memory(h);
     }
-    return join(h);
+    return join_through_memory(h);
 }
 
 extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, int N, int K,
@@ -340,7 +332,7 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
         }
         i = j;
     }
-    return fused ? join(h) : join_through_memory(h);
+    return join_through_memory(h);
 }
 
 extern "C" int fo_overlap_gemm_allreduce_serial(fo_overlap_t *h, int dtype, int M, int N, int K,
