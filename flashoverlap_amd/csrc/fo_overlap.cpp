@@ -1,6 +1,6 @@
 // Host orchestration of the overlap path: the counterpart of class OverlapImpl
 // (src/overlap_impl.h:12-43, src/overlap_impl.cu) behind a C handle.  Two HIP
-// streams and one event; every call only enqueues work and returns.
+// streams; every call only enqueues work and returns.
 #include <new>
 
 #include "fo_common.h"
@@ -8,7 +8,6 @@
 struct fo_overlap {
     hipStream_t gemm_stream = nullptr;
     hipStream_t comm_stream = nullptr;
-    hipEvent_t forked = nullptr;
     int32_t *workspace = nullptr;  // zeroed words of the one-launch wait+reduce kernel
     bool gemm_ready = false;
     bool overlap_ready = false;
@@ -77,15 +76,16 @@ int check_segments(const int32_t *cseg_host, int G, long tiles) {
     return sum == tiles ? FO_OK : FO_ERR_SEGMENTS;
 }
 
-// GEMM stream -> consumer stream, recorded right before the GEMM is enqueued.  Only the
+// GEMM stream -> consumer stream, right before the GEMM is enqueued (through memory, like
+// the join below: a one-lane set on the GEMM stream, a one-lane wait on the other).  Only the
 // one-launch consumer needs it: its workgroups poll from the moment they start, and polls
 // slow down whatever shares the memory system with them, so they must not start while the
 // GEMM stream is still busy with the work that precedes the GEMM (the reference's wait
 // kernels may start early: a single sleeping lane disturbs nobody).
 int fork(fo_overlap *h) {
-    FO_HIP_CHECK(hipEventRecord(h->forked, h->gemm_stream));
-    FO_HIP_CHECK(hipStreamWaitEvent(h->comm_stream, h->forked, 0));
-    return FO_OK;
+    int rc = fo_set(h->workspace + 5, 1, h->gemm_stream);
+    if (rc) return rc;
+    return fo_wait(1, h->workspace + 5, h->comm_stream);
 }
 
 // consumer stream -> GEMM stream.  The reference records an event on the consumer stream
@@ -132,7 +132,6 @@ extern "C" int fo_overlap_destroy(fo_overlap_t *h) {
         hipStreamSynchronize(h->comm_stream);
         hipStreamDestroy(h->comm_stream);
     }
-    if (h->forked) hipEventDestroy(h->forked);
     if (h->workspace) hipFree(h->workspace);
     delete h;
     return FO_OK;
@@ -151,7 +150,6 @@ extern "C" int fo_overlap_init(fo_overlap_t *h) {
     // Default priority on purpose (the reference asks for priority -5,
     // src/overlap_impl.cu:140): mixed-priority streams are avoided on this platform.
     FO_HIP_CHECK(hipStreamCreateWithFlags(&h->comm_stream, hipStreamNonBlocking));
-    FO_HIP_CHECK(hipEventCreateWithFlags(&h->forked, hipEventDisableTiming));
     FO_HIP_CHECK(hipMalloc(&h->workspace, 64));
     FO_HIP_CHECK(hipMemset(h->workspace, 0, 64));
     h->overlap_ready = true;
