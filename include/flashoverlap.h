@@ -223,8 +223,10 @@ fo_stream_t fo_overlap_comm_stream(fo_overlap_t *h);
 int fo_overlap_gemm(fo_overlap_t *h, int dtype, int M, int N, int K, const void *A, const void *B,
                     void *C, int algo);
 /* GemmAllReduceOverlap(...), src/overlap_impl.cu:214-264: signal GEMM on the
- * GEMM stream; per group {wait, consume} on the consumer stream; event join
- * consumer -> GEMM stream.  cseg_host[G] is host memory. */
+ * GEMM stream; per group {wait, consume} on the consumer stream (groups of one
+ * GEMM wave share a launch, see fo_overlap_plan_batches); then the GEMM stream
+ * is made to wait for the consumer stream, through memory (fo_set / fo_wait)
+ * where the reference uses an event pair.  cseg_host[G] is host memory. */
 int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int N, int K, const void *A,
                               const void *B, void *C, int32_t *MM, const int32_t *RA, int TM,
                               int TN, int rLDN, const int32_t *cseg_host,
