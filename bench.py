@@ -49,6 +49,9 @@ def main():
     ap.add_argument("--kernels-only", action="store_true",
                     help="run each hot kernel alone on one stream and exit: for counter collection, which "
                          "serialises dispatches and would stall a waiter that spins on another queue")
+    ap.add_argument("--steps-only", action="store_true",
+                    help="enqueue warmup + steps overlapped steps and exit: for a kernel-trace timeline of the "
+                         "steady state")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a 256 MiB device-to-device copy five times (reference point for "
                          "scaling the FETCH_SIZE / WRITE_SIZE counters) and exit")
@@ -170,6 +173,10 @@ def main():
         return e0.elapsed_time(e1) / steps, wall
 
     K_, W_ = args.steps, args.warmup
+    if args.steps_only:
+        ms, _ = timed(step_overlapped, K_, W_)
+        print(json.dumps({"steps_only": True, "steps": K_, "warmup": W_, "ms_per_step": ms}))
+        return
     if args.kernels_only:
         for fn in (gemm_alone, gemm_signal_alone, consumer_alone, norm):
             timed(fn, K_, W_)
