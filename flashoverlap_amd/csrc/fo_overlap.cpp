@@ -128,13 +128,18 @@ extern "C" int fo_overlap_create(fo_overlap_t **out) {
 
 extern "C" int fo_overlap_destroy(fo_overlap_t *h) {
     if (!h) return FO_ERR_ARG;
+    // release everything even if one step fails; report the first failure
+    hipError_t first = hipSuccess;
+    auto note = [&](hipError_t e) {
+        if (first == hipSuccess) first = e;
+    };
     if (h->comm_stream) {
-        hipStreamSynchronize(h->comm_stream);
-        hipStreamDestroy(h->comm_stream);
+        note(hipStreamSynchronize(h->comm_stream));
+        note(hipStreamDestroy(h->comm_stream));
     }
-    if (h->workspace) hipFree(h->workspace);
+    if (h->workspace) note(hipFree(h->workspace));
     delete h;
-    return FO_OK;
+    return (int)first;
 }
 
 extern "C" int fo_overlap_set_gemm_stream(fo_overlap_t *h, fo_stream_t gemm_stream) {
