@@ -1,6 +1,6 @@
 // Host orchestration of the overlap path: the counterpart of class OverlapImpl
 // (src/overlap_impl.h:12-43, src/overlap_impl.cu) behind a C handle.  Two HIP
-// streams; every call only enqueues work and returns.
+// streams; every call only enqueues work and returns.  May be captured into a HIP graph.
 #include <new>
 
 #include "fo_common.h"
@@ -8,6 +8,7 @@
 struct fo_overlap {
     hipStream_t gemm_stream = nullptr;
     hipStream_t comm_stream = nullptr;
+    hipEvent_t forked = nullptr, joined = nullptr;  // used only while the GEMM stream is being captured
     int32_t *workspace = nullptr;  // zeroed words of the one-launch wait+reduce kernel
     bool gemm_ready = false;
     bool overlap_ready = false;
@@ -76,13 +77,29 @@ int check_segments(const int32_t *cseg_host, int G, long tiles) {
     return sum == tiles ? FO_OK : FO_ERR_SEGMENTS;
 }
 
-// GEMM stream -> consumer stream, right before the GEMM is enqueued (through memory, like
-// the join below: a one-lane set on the GEMM stream, a one-lane wait on the other).  Only the
-// one-launch consumer needs it: its workgroups poll from the moment they start, and polls
-// slow down whatever shares the memory system with them, so they must not start while the
-// GEMM stream is still busy with the work that precedes the GEMM (the reference's wait
-// kernels may start early: a single sleeping lane disturbs nobody).
-int fork(fo_overlap *h) {
+// While the GEMM stream is being captured into a HIP graph the two streams are tied
+// together with events, as in the reference (src/overlap_impl.cu:246, :260-263): the
+// event wait pulls the consumer stream into the capture, and in the graph the dependency
+// is an edge, not a wait at run time.
+bool capturing(const fo_overlap *h) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(h->gemm_stream, &st) != hipSuccess) return false;
+    return st == hipStreamCaptureStatusActive;
+}
+
+// GEMM stream -> consumer stream, right before the GEMM is enqueued.  Outside a capture it
+// goes through memory (a one-lane set on the GEMM stream, a one-lane wait on the other) and
+// only the one-launch consumer needs it: its workgroups poll from the moment they start,
+// and polls slow down whatever shares the memory system with them, so they must not start
+// while the GEMM stream is still busy with the work that precedes the GEMM (the
+// reference's wait kernels may start early: a single sleeping lane disturbs nobody).
+int fork(fo_overlap *h, bool captured, bool polling_consumer) {
+    if (captured) {
+        FO_HIP_CHECK(hipEventRecord(h->forked, h->gemm_stream));
+        FO_HIP_CHECK(hipStreamWaitEvent(h->comm_stream, h->forked, 0));
+        return FO_OK;
+    }
+    if (!polling_consumer) return FO_OK;
     int rc = fo_set(h->workspace + 5, 1, h->gemm_stream);
     if (rc) return rc;
     return fo_wait(1, h->workspace + 5, h->comm_stream);
@@ -90,13 +107,18 @@ int fork(fo_overlap *h) {
 
 // consumer stream -> GEMM stream.  The reference records an event on the consumer stream
 // and makes the GEMM stream wait for it (src/overlap_impl.cu:260-263); an event wait across
-// queues measured about 12 us here, so the join goes through memory instead: a one-lane
-// kernel at the end of the consumer stream sets workspace word 4 (stream order makes all
-// earlier work there complete and visible first), a one-lane wait behind the GEMM on the
-// GEMM's stream consumes it.  The wait cannot start before the GEMM has ended and
-// everything it waits for was enqueued before it; the GEMM stream continues about 4 us
+// queues measured about 12 us here, so outside a capture the join goes through memory: a
+// one-lane kernel at the end of the consumer stream sets workspace word 4 (stream order
+// makes all earlier work there complete and visible first), a one-lane wait behind the
+// GEMM on the GEMM's stream consumes it.  The wait cannot start before the GEMM has ended
+// and everything it waits for was enqueued before it; the GEMM stream continues about 4 us
 // after the consumer's end.
-int join_through_memory(fo_overlap *h) {
+int join(fo_overlap *h, bool captured) {
+    if (captured) {
+        FO_HIP_CHECK(hipEventRecord(h->joined, h->comm_stream));
+        FO_HIP_CHECK(hipStreamWaitEvent(h->gemm_stream, h->joined, 0));
+        return FO_OK;
+    }
     int rc = fo_set(h->workspace + 4, 1, h->comm_stream);
     if (rc) return rc;
     return fo_wait(1, h->workspace + 4, h->gemm_stream);
@@ -137,6 +159,8 @@ extern "C" int fo_overlap_destroy(fo_overlap_t *h) {
         note(hipStreamSynchronize(h->comm_stream));
         note(hipStreamDestroy(h->comm_stream));
     }
+    if (h->forked) note(hipEventDestroy(h->forked));
+    if (h->joined) note(hipEventDestroy(h->joined));
     if (h->workspace) note(hipFree(h->workspace));
     delete h;
     return (int)first;
@@ -155,6 +179,8 @@ extern "C" int fo_overlap_init(fo_overlap_t *h) {
     // Default priority on purpose (the reference asks for priority -5,
     // src/overlap_impl.cu:140): mixed-priority streams are avoided on this platform.
     FO_HIP_CHECK(hipStreamCreateWithFlags(&h->comm_stream, hipStreamNonBlocking));
+    FO_HIP_CHECK(hipEventCreateWithFlags(&h->forked, hipEventDisableTiming));
+    FO_HIP_CHECK(hipEventCreateWithFlags(&h->joined, hipEventDisableTiming));
     FO_HIP_CHECK(hipMalloc(&h->workspace, 64));
     FO_HIP_CHECK(hipMemset(h->workspace, 0, 64));
     h->overlap_ready = true;
@@ -215,10 +241,9 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
         rc = fo_gemm_wave_tiles(dtype, algo, M, N, &wave);
         if (rc) return rc;
     }
-    if (fused) {
-        rc = fork(h);
-        if (rc) return rc;
-    }
+    const bool captured = capturing(h);
+    rc = fork(h, captured, fused != 0);
+    if (rc) return rc;
     rc = fo_gemm_signal(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, MM, RA, monitor, algo,
                         h->gemm_stream);
     if (rc) return rc;  // nothing has been enqueued on the consumer stream yet
@@ -250,7 +275,7 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
             i = j;
         }
     }
-    return join_through_memory(h);
+    return join(h, captured);
 }
 
 extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, int N, int K,
@@ -279,10 +304,9 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
         rc = fo_gemm_wave_tiles(dtype, algo, M, N, &wave);
         if (rc) return rc;
     }
-    if (fused) {
-        rc = fork(h);
-        if (rc) return rc;
-    }
+    const bool captured = capturing(h);
+    rc = fork(h, captured, fused != 0);
+    if (rc) return rc;
     rc = fo_gemm_scatter(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, MM, RA, RE, monitor, algo,
                          h->gemm_stream);
     if (rc) return rc;
@@ -335,7 +359,7 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
         }
         i = j;
     }
-    return join_through_memory(h);
+    return join(h, captured);
 }
 
 extern "C" int fo_overlap_gemm_allreduce_serial(fo_overlap_t *h, int dtype, int M, int N, int K,

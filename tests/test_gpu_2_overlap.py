@@ -421,3 +421,55 @@ def test_uneven_tile_walk_matches_vendor_gemm(fo):
     torch.cuda.synchronize()
     assert MM[:len(cseg)].tolist() == cseg
     assert torch.equal(fo.layout.unpermute(Cp, M, N, bm, bn, RA), C)
+
+
+@pytest.mark.parametrize("fused", [0, 1])
+def test_overlapped_step_captured_in_a_hip_graph(fo, fused):
+    """Capture {overlapped GEMM + consumer, reorder+RMSNorm} once, replay it several times with eager
+    work and synchronisations in between and new operand values each time; every replay must give
+    what the eager path gives.  Under capture the two streams are tied by events (graph edges)."""
+    M, N, K, bm, bn = 2048, 2048, 256, 128, 128
+    cseg = [64] * 4
+    algo, RA, A, B, _, _, MM, cs_cpu, cs_gpu = _setup(fo, F16, bm, bn, M, N, K, cseg, swizzle=4, seed=120)
+    ops = fo.ops
+    Cp = torch.empty(M * N, device="cuda", dtype=torch.float16)
+    ACC = torch.zeros(M * N, device="cuda", dtype=torch.float16)
+    Y = torch.empty(M, N, device="cuda", dtype=torch.float16)
+    gamma = (1 + 0.01 * torch.randn(N, device="cuda")).half()
+    A0 = A.clone()
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        ov = ops.Overlap()                    # GEMM stream = s
+        ov.set_accumulator(ACC)
+        ov.set_fused_consumer(fused)
+
+        def step():
+            ov.gemm_allreduce_overlap(A, B, Cp, MM, RA, 1, cs_cpu, cs_gpu, algo)
+            ops.reorder_rmsnorm(Cp.view(M, N), Y, gamma, bm, bn, 1, RA, eps=1e-6)
+
+        step()                                # eager warm-up: one-time kernel attribute set-up
+    torch.cuda.synchronize()
+    ACC.zero_()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=s):
+        step()
+    torch.cuda.synchronize()
+    ACC.zero_()                               # whatever the capture pass itself did not run
+
+    plain = torch.empty(M, N, device="cuda", dtype=torch.float16)
+    y_ref = torch.empty_like(Y)
+    expect = torch.zeros(M * N, device="cuda", dtype=torch.float32)
+    for it in range(4):
+        A.copy_((A0 * (0.5 + 0.25 * it)).roll(it * 11, dims=1))       # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        ops.gemm(A, B, plain, algo)
+        ops.rmsnorm(plain, y_ref, gamma, eps=1e-6)
+        torch.cuda.synchronize()
+        assert torch.equal(fo.layout.unpermute(Cp, M, N, bm, bn, RA), plain), f"replay {it}"
+        assert torch.equal(Y, y_ref), f"replay {it}"
+        expect = (expect + Cp.float()).half().float()
+        assert torch.equal(ACC.float(), expect), f"replay {it}"
+        assert (MM == 0).all()
+    ov.close()
