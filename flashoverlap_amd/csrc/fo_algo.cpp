@@ -110,7 +110,7 @@ extern "C" const char *fo_error_string(int code) {
     switch (code) {
         case FO_OK: return "ok";
         case FO_ERR_ARG: return "null pointer or non-positive size";
-        case FO_ERR_SHAPE: return "shape not divisible by the tile (M % BM, N % BN, K % 64, dim % 8)";
+        case FO_ERR_SHAPE: return "shape not divisible by the tile (M % BM, N % BN, K % 8, dim % 8)";
         case FO_ERR_ALGO: return "Algo index out of range";
         case FO_ERR_DTYPE: return "dtype must be FO_F16 or FO_BF16";
         case FO_ERR_SEGMENTS: return "cSeg does not partition the tiles (or too many groups for monitor mode)";

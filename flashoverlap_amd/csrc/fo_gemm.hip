@@ -75,7 +75,7 @@ int run_gemm(int mode, int dtype, int M, int N, int K, int rLDN, const int32_t *
     fo_raster r;
     int rc = fo_pick_raster(algo, M, N, &r);
     if (rc) return rc;
-    if (K % 64) return FO_ERR_SHAPE;
+    if (K % 8) return FO_ERR_SHAPE;  // operand rows are fetched in 16-byte chunks
     // the epilogue assumes a wavefront's 128 x 64 (or 64 x 64) block lies inside one reorder tile
     if (e->f[0] % 128 || e->f[1] % 128) return FO_ERR_ALGO;
     GemmArgs a;

@@ -173,7 +173,12 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
     const int ntiles = p.grid_m * p.grid_n;
-    const int KT = p.K / BK;
+    // K is a multiple of 8 (one 16-byte chunk).  A last K step that is not full
+    // is loaded with its out-of-range chunks redirected to the step's first
+    // chunk (valid memory) and zeroed in LDS before the stage is published.
+    const int KT = (p.K + BK - 1) / BK;
+    const bool ktail = (p.K % BK) != 0;
+    const int KT_full = ktail ? KT - 1 : KT;  // K steps whose loads need no special care
 
     // Fragment addressing: lane l supplies row (l & 31), k-chunk (l >> 5) of
     // each 32x16 operand block.
@@ -203,14 +208,52 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
         Bb = (gptr_t)(p.B) + ((size_t)pn_ * MTN + wave * (64 / CH)) * p.ldb * 2;
     };
     // Issue the loads of K step kt into ring slot s (P instructions per wavefront).
-    auto issue = [&](int kt, int s) {
+    auto issue_with = [&](int kt, int s, unsigned al, unsigned bl) {
         const unsigned as = smem_lds + (unsigned)(s * STAGE16 + wave * 64) * 16;  // LDS byte addresses
         const unsigned bs = as + MTM * CH * 16;
         gptr_t ak = Ab + (size_t)kt * (BK * 2), bk = Bb + (size_t)kt * (BK * 2);
 #pragma unroll
-        for (int i = 0; i < PA; i++) dma_load16(ak + i * a_blk_bytes, a_lane, as + i * NW * 1024);
+        for (int i = 0; i < PA; i++) dma_load16(ak + i * a_blk_bytes, al, as + i * NW * 1024);
 #pragma unroll
-        for (int i = 0; i < PB; i++) dma_load16(bk + i * b_blk_bytes, b_lane, bs + i * NW * 1024);
+        for (int i = 0; i < PB; i++) dma_load16(bk + i * b_blk_bytes, bl, bs + i * NW * 1024);
+    };
+    auto issue = [&](int kt, int s) { issue_with(kt, s, a_lane, b_lane); };
+    // The partial last K step.  Whether this lane's chunk lies beyond K is
+    // recomputed from a laundered lane id, so nothing of it stays live across
+    // the K loop.
+    auto tail_chunk_out = [&](int *row) {
+        int el = lane;
+        asm volatile("" : "+v"(el));
+        *row = el / CH;
+        const int lc = (el % CH) ^ (((wave * (64 / CH) + el / CH) >> SWZ_SHIFT) & (CH - 1));
+        return (KT - 1) * BK + lc * 8 >= p.K;
+    };
+    // Same loads as issue(); a chunk beyond K is fetched from the row's first chunk of this step instead.
+    auto issue_any = [&](int kt, int s) {
+        if (ktail && kt == KT - 1) {
+            int row;
+            const bool out = tail_chunk_out(&row);
+            issue_with(kt, s, out ? (unsigned)(row * p.lda * 2) : a_lane, out ? (unsigned)(row * p.ldb * 2) : b_lane);
+        } else {
+            issue(kt, s);
+        }
+    };
+    // Zero this lane's chunks of the partial step in ring slot s.  Called after
+    // the lane's own loads of that stage have landed and before the barrier that
+    // publishes the stage.
+    auto zero_tail = [&](int s) {
+        int row;
+        if (tail_chunk_out(&row)) {
+            int el = lane;
+            asm volatile("" : "+v"(el));
+            fo_u32x4 *mine = smem + s * STAGE16 + wave * 64 + el;
+            const fo_u32x4 z = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int i = 0; i < PA; i++) mine[i * NW * 64] = z;
+#pragma unroll
+            for (int i = 0; i < PB; i++) mine[MTM * CH + i * NW * 64] = z;
+        }
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
     };
 
     // ---- signalling state (signal and scatter epilogues)
@@ -307,12 +350,19 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
                     wait_vmcnt<(STAGES - 2) * P>();
                 else
                     wait_vmcnt<0>();
+                if (!STEADY) {
+                    if (ktail && kt + 2 == KT) zero_tail(nslot);  // all loads of stage KT-1 have landed (vmcnt 0)
+                }
                 __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
                 if (!STEADY && MODE != MODE_PLAIN) {
                     if (first && owed && wave == 0) announce(prev_rs);
                 }
-                if (STEADY || kt + STAGES < KT) issue(kt + STAGES, slot);
+                if constexpr (STEADY) {
+                    issue(kt + STAGES, slot);
+                } else {
+                    if (kt + STAGES < KT) issue_any(kt + STAGES, slot);
+                }
                 FO_LOAD_FRAGS((kk + 1) & 1, smem + nslot * STAGE16, 0)
             }
             FO_MFMAS(kk)
@@ -339,7 +389,7 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
     pm = __builtin_amdgcn_readfirstlane(pm);
     pn = __builtin_amdgcn_readfirstlane(pn);
     set_tile(pm, pn);
-    issue(0, 0);
+    issue_any(0, 0);
     bool carried = false;  // stores of an earlier tile may still be in flight
 
     for (;;) {
@@ -365,20 +415,22 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
         if (!carried) {
 #pragma unroll
             for (int s = 1; s < STAGES; s++)
-                if (s < KT) issue(s, s);
+                if (s < KT) issue_any(s, s);
             if (KT >= STAGES)
                 wait_vmcnt<(STAGES - 1) * P>();
             else
                 wait_vmcnt<0>();
+            if (ktail && KT == 1) zero_tail(0);
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
         } else {
             wait_vmcnt<NST>();
+            if (ktail && KT == 1) zero_tail(0);
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
 #pragma unroll
             for (int s = 1; s < STAGES; s++)
-                if (s < KT) issue(s, s);
+                if (s < KT) issue_any(s, s);
         }
         FO_LOAD_FRAGS(0, smem, 0)
 
@@ -393,12 +445,12 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
         if (MODE != MODE_PLAIN && KT >= 2) owed = false;  // sent in the first K step
         if constexpr (STAGES == 2) {
             // here kt == 1 (slot 1) when KT > 1
-            for (; kt + 1 + STAGES < KT; kt += 2) {
+            for (; kt + 1 + STAGES < KT_full; kt += 2) {
                 kstep(std::true_type{}, std::integral_constant<int, 1>{}, false, kt, 1, 0);
                 kstep(std::true_type{}, std::integral_constant<int, 0>{}, false, kt + 1, 0, 1);
             }
         } else {
-            for (; kt + STAGES < KT; kt++) {
+            for (; kt + STAGES < KT_full; kt++) {
                 const int nslot = slot + 1 == STAGES ? 0 : slot + 1;
                 kstep(std::true_type{}, dyn{}, false, kt, slot, nslot);
                 slot = nslot;
@@ -424,7 +476,7 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
             pm = __builtin_amdgcn_readfirstlane(pm);
             pn = __builtin_amdgcn_readfirstlane(pn);
             set_tile(pm, pn);
-            issue(0, 0);
+            issue_any(0, 0);
         }
 
         // ---- epilogue: accumulators -> 16-bit -> LDS (per-wave strip of 32 rows) -> global

@@ -29,7 +29,7 @@ enum { FO_F16 = 0, FO_BF16 = 1 };
 enum {
     FO_OK = 0,
     FO_ERR_ARG = -1,      /* null pointer / non-positive size */
-    FO_ERR_SHAPE = -2,    /* M % BM, N % BN, K % 64, dim % 8 ... violated */
+    FO_ERR_SHAPE = -2,    /* M % BM, N % BN, K % 8, dim % 8 ... violated */
     FO_ERR_ALGO = -3,     /* Algo outside [0, fo_algo_count()) */
     FO_ERR_DTYPE = -4,    /* dtype not FO_F16 / FO_BF16 */
     FO_ERR_SEGMENTS = -5, /* sum(cSeg) != tile count, G <= 0, monitor with G > TN-1 */
@@ -70,8 +70,9 @@ int fo_gemm_wave_tiles(int dtype, int algo, int M, int N, int32_t *tiles);
  * C[M,N] = A[M,K] . B[N,K]^T, 16-bit in/out, fp32 accumulate.
  * Replaces gemm_func_table[Algo](M,N,K,A,B,C,stream), src/gemm/gemm.cu:23-110,
  * typedef src/tiling/gemm_dispatcher.h:7-26. Requires M % TbM == 0,
- * N % TbN == 0, K % 64 == 0 (the reference has no boundary handling either,
- * README.md:73). */
+ * N % TbN == 0 (the reference has no boundary handling either, README.md:73)
+ * and K % 8 == 0 (rows are fetched in 16-byte pieces; a last K step that is not
+ * full is zero-filled on chip). */
 int fo_gemm(int dtype, int M, int N, int K, const void *A, const void *B, void *C, int algo,
             fo_stream_t stream);
 

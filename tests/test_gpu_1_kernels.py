@@ -131,6 +131,43 @@ def test_signal_gemm_persistent_walk(fo, oracle):
     _signal_case(fo, oracle, F16, 128, 128, 4224, 4224, 64, [1] * 1089)
 
 
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("bm,bn,M,N,K", [(128, 128, 256, 384, 8), (128, 128, 256, 384, 72),
+                                         (128, 128, 384, 256, 200), (128, 128, 256, 256, 1376),
+                                         (128, 256, 256, 512, 104), (256, 128, 512, 256, 136),
+                                         (128, 256, 256, 512, 24), (128, 128, 4352, 4096, 88)])
+def test_gemm_partial_last_k_step(fo, oracle, dtype, bm, bn, M, N, K):
+    """K is any multiple of 8: the chunks of the last K step that lie beyond K are zero-filled on
+    chip.  The operands end exactly at the end of a buffer whose tail is NaN, so a read past a
+    row's end that reached the accumulators would show (it would bring the next row's head, or
+    the NaN tail for the last row)."""
+    t = TORCH_DTYPE[dtype]
+    A, Ab = seeded((M, K), dtype, 31)
+    B, Bb = seeded((N, K), dtype, 32, scale=K ** -0.5)
+    bufA = torch.full((M * K + 256,), float("nan"), device="cuda", dtype=t)
+    bufB = torch.full((N * K + 256,), float("nan"), device="cuda", dtype=t)
+    bufA[:M * K] = A.reshape(-1)
+    bufB[:N * K] = B.reshape(-1)
+    C = torch.empty(M, N, device="cuda", dtype=t)
+    fo.ops.gemm(bufA[:M * K].view(M, K), bufB[:N * K].view(N, K), C, _algo(fo, bm, bn))
+    torch.cuda.synchronize()
+    ref_bits, _ = oracle.gemm_signal(dtype, Ab, Bb, bm, bn)
+    ref = torch.from_numpy(oracle.from_bits(ref_bits, dtype))
+    assert not torch.isnan(C).any()
+    assert max_rel_err(C.float().cpu(), ref) <= REL_TOL
+    assert ulp_diff_ok(bits_of(C), ref_bits, dtype, max_ulp=1, frac=0.999)
+
+
+def test_signal_gemm_partial_last_k_step(fo, oracle):
+    """The partial K step inside the persistent walk: as a tile's only step (requested before
+    the previous tile's epilogue), as the second of two, and behind the steady loop."""
+    _signal_case(fo, oracle, F16, 128, 128, 3200, 3072, 40, [300, 300])
+    _signal_case(fo, oracle, BF16, 128, 128, 3200, 3072, 72, [599, 1])
+    _signal_case(fo, oracle, F16, 128, 128, 4352, 4096, 456, [272] * 4, swizzle=4)
+    _signal_case(fo, oracle, F16, 256, 128, 4352, 4096, 200, [300, 244], swizzle=4, W=2)
+    _signal_case(fo, oracle, F16, 128, 256, 1024, 1024, 328, [16, 16])
+
+
 def test_scatter_gemm_row_map(fo, oracle):
     _signal_case(fo, oracle, F16, 128, 128, 512, 512, 64, [4, 4, 8], W=4)
     _signal_case(fo, oracle, BF16, 128, 128, 512, 256, 128, [3, 5], W=8)

@@ -67,7 +67,7 @@ def test_argument_validation_without_gpu():
     one = ctypes.c_void_p(16)  # never dereferenced: validation fails first
     assert L.fo_gemm(0, 128, 128, 64, null, one, one, 0, null) == -1           # null A
     assert L.fo_gemm(0, 100, 128, 64, one, one, one, 0, null) == -2            # M % 128
-    assert L.fo_gemm(0, 128, 128, 70, one, one, one, 0, null) == -2            # K % 64
+    assert L.fo_gemm(0, 128, 128, 68, one, one, one, 0, null) == -2            # K % 8
     assert L.fo_gemm(0, 128, 128, 64, one, one, one, 102, null) == -3          # Algo range
     assert L.fo_gemm(7, 128, 128, 64, one, one, one, 0, null) == -4            # dtype
     assert L.fo_gemm_signal(0, 128, 128, 64, 1, one, 0, one, one, one, one, one, 0, 0, null) == -5
