@@ -22,7 +22,7 @@
 
 typedef _Float16 fo_half8 __attribute__((ext_vector_type(8)));
 typedef __bf16 fo_bf8 __attribute__((ext_vector_type(8)));
-typedef float fo_float16v __attribute__((ext_vector_type(16)));
+typedef float fo_float4v __attribute__((ext_vector_type(4)));
 // Native 16- and 8-byte vectors (HIP's uint4 is a struct that register promotion handles badly).
 typedef unsigned int fo_u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int fo_u32x2 __attribute__((ext_vector_type(2)));
@@ -41,9 +41,17 @@ template <> struct fo_elem<fo_f16_tag> {
     static __device__ __forceinline__ uint16_t from_f32(float f) {
         return __builtin_bit_cast(uint16_t, (_Float16)f);
     }
-    static __device__ __forceinline__ fo_float16v mfma(fo_u32x4 a, fo_u32x4 b, fo_float16v c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(fo_half8, a),
-                                                      __builtin_bit_cast(fo_half8, b), c, 0, 0, 0);
+    // D(16x16) += A(16x32) . B(32x16); lane l supplies row l & 15, k-chunk l >> 4 of both
+    // operands and holds D[4 * (l >> 4) + v][l & 15], v = 0..3.
+    // Written as assembly with the accumulator tied to the destination: the
+    // builtin's destination is a free operand for this shape, and with 32
+    // accumulator blocks in a doubly unrolled loop the register allocator then
+    // rotates them through spare registers and spills.  What the compiler
+    // therefore does not see is that the result is late: callers keep VALU reads
+    // and writes of the accumulators (zeroing, conversion) 24 wait states away
+    // from these instructions (fo_mfma_fence).
+    static __device__ __forceinline__ void mfma(fo_u32x4 a, fo_u32x4 b, fo_float4v &c) {
+        asm("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
     }
 };
 template <> struct fo_elem<fo_bf16_tag> {
@@ -55,11 +63,18 @@ template <> struct fo_elem<fo_bf16_tag> {
     static __device__ __forceinline__ uint16_t from_f32(float f) {
         return __builtin_bit_cast(uint16_t, (__bf16)f);
     }
-    static __device__ __forceinline__ fo_float16v mfma(fo_u32x4 a, fo_u32x4 b, fo_float16v c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(fo_bf8, a),
-                                                       __builtin_bit_cast(fo_bf8, b), c, 0, 0, 0);
+    static __device__ __forceinline__ void mfma(fo_u32x4 a, fo_u32x4 b, fo_float4v &c) {
+        asm("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
     }
 };
+
+// Wait states between the assembly MFMAs and ordinary VALU code touching their
+// accumulators (longest case: an 8-pass MFMA result read by a VALU instruction).
+static __device__ __forceinline__ void fo_mfma_fence() {
+    __builtin_amdgcn_sched_barrier(0);  // nothing is scheduled across the wait states
+    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
 
 // Algo table (fo_algo.cpp).
 struct fo_algo_entry {

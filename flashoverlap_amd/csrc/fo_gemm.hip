@@ -12,10 +12,10 @@ using namespace fo_gemm_dev;
 // fewer macro tiles); each walks the raster with that stride.
 // With `resident_out` set nothing is launched: the call only reports how many workgroups the
 // launch would hold.
-template <typename Tag, int MTM, int MTN, int BK, int STAGES, int WM, int WN, int MODE>
+template <typename Tag, int MTM, int MTN, int BK, int SA, int SB, int WM, int WN, int MODE>
 int launch_variant(const GemmArgs &a, hipStream_t stream, int *resident_out) {
-    auto kern = fo_gemm_kernel<Tag, MTM, MTN, BK, STAGES, WM, WN, MODE>;
-    constexpr int smem = smem_bytes<MTM, MTN, BK, STAGES>();
+    auto kern = fo_gemm_kernel<Tag, MTM, MTN, BK, SA, SB, WM, WN, MODE>;
+    constexpr int smem = smem_bytes<MTM, MTN, BK, SA, SB>();
     constexpr int threads = WM * WN * 64;
     static int resident = 0;  // per instantiation; the attribute is process wide
     if (!resident) {
@@ -42,19 +42,19 @@ int launch_variant(const GemmArgs &a, hipStream_t stream, int *resident_out) {
     return FO_OK;
 }
 
-// Macro tile -> kernel shape.  256x256 (eight wavefronts, two LDS slots of
-// 64 KiB) is the workhorse; the smaller shapes serve problems whose M or N is
+// Macro tile -> kernel shape.  256x256 (eight wavefronts, three 32 KiB slots for
+// the A part and two for the B part of a K step: all 160 KiB) is the workhorse; the smaller shapes serve problems whose M or N is
 // not a multiple of 256 or that have too few 256x256 tiles to fill the chip.
 template <typename Tag, int MODE>
 int launch_tile(const GemmArgs &a, int mtm, int mtn, hipStream_t stream, int *resident_out) {
     if (mtm == 256 && mtn == 256)
-        return launch_variant<Tag, 256, 256, 64, 2, 2, 4, MODE>(a, stream, resident_out);
+        return launch_variant<Tag, 256, 256, 64, 2, 2, 2, 4, MODE>(a, stream, resident_out);
     if (mtm == 128 && mtn == 128)
-        return launch_variant<Tag, 128, 128, 64, 2, 2, 2, MODE>(a, stream, resident_out);
+        return launch_variant<Tag, 128, 128, 64, 2, 2, 2, 2, MODE>(a, stream, resident_out);
     if (mtm == 128 && mtn == 256)
-        return launch_variant<Tag, 128, 256, 64, 3, 2, 4, MODE>(a, stream, resident_out);
+        return launch_variant<Tag, 128, 256, 64, 3, 3, 2, 4, MODE>(a, stream, resident_out);
     if (mtm == 256 && mtn == 128)
-        return launch_variant<Tag, 256, 128, 64, 3, 2, 2, MODE>(a, stream, resident_out);
+        return launch_variant<Tag, 256, 128, 64, 3, 3, 2, 2, MODE>(a, stream, resident_out);
     return FO_ERR_ALGO;
 }
 

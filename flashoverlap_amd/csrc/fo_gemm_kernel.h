@@ -12,15 +12,24 @@
 // The kernel is persistent: the launch holds at most as many workgroups as the
 // chip keeps resident, and workgroup w computes macro tiles w, w + grid,
 // w + 2 grid, ... of the raster.  A workgroup of WM x WN wavefronts computes an
-// MTM x MTN macro tile with v_mfma_f32_32x32x16_{f16,bf16}.  Operand tiles of
-// BK columns travel HBM -> LDS directly (global_load_lds_dwordx4, 1 KiB per
-// wavefront instruction, no VGPR staging) into a ring of STAGES buffers; a slot
-// is recycled as soon as every wavefront holds its last fragments of it in
-// registers; one s_barrier per K step.  The 16-byte chunks of a tile row are
-// XOR-swizzled (by choosing which global chunk each lane fetches) so that the
-// 16 lanes a ds_read_b128 serves per clock hit 16 different bank groups.  The
-// accumulators leave through LDS so that every global store is a 16-byte piece
-// of a contiguous output row.
+// MTM x MTN macro tile with v_mfma_f32_16x16x32_{f16,bf16}: in an MFMA-only
+// loop under this part's power limit that form sustains 14 % more than
+// 32x32x16 (a quarter of the accumulator registers per instruction, half of
+// their traffic per flop), and the whole kernel is power-limited.
+//
+// Operand tiles of BK columns travel HBM -> LDS directly
+// (global_load_lds_dwordx4, 1 KiB per wavefront instruction, no VGPR staging)
+// into two rings, SA slots for the A part of a K step and SB <= SA slots for
+// the B part; one s_barrier per K step, placed behind the last LDS read of the
+// step, recycles both slots.  (SA = SB + 1 = 3 is all that 160 KiB of LDS allow
+// for a 256x256x64 step: the A part is then requested two K steps ahead.  It
+// measured 4 % faster with all-zero operands and no faster with real ones, and
+// is not used.)  The 16-byte chunks of a tile row are XOR-swizzled (by choosing
+// which global chunk each lane fetches) so that the 16 lanes a ds_read_b128
+// serves per clock hit 16 different bank groups.  Fragments stream through a
+// short register ring (see the K step), 32 accumulator blocks of 16x16 stay in
+// place, and the accumulators leave through LDS so that every global store is
+// a 16-byte piece of a contiguous output row.
 //
 // Tile i+1's first operand stage is requested before tile i's epilogue and
 // lands while the epilogue runs; tile i's completion signal is sent from inside
@@ -53,7 +62,7 @@ struct GemmArgs {
 };
 
 constexpr int kMaxSub = 4;        // reorder tiles per macro tile (256x256 over 128x128)
-constexpr int kPrefixMax = 1024;  // group search on an LDS table for up to this many groups
+constexpr int kPrefixRegs = 128;  // group search on prefix sums held in two registers per lane up to this many groups
 
 // Group of storage slot r: smallest g with cseg[0]+..+cseg[g] > r
 // (src/overlap/gemm_with_signal.h:343-349), found by one wavefront with a
@@ -74,18 +83,6 @@ __device__ __forceinline__ int find_group(const int32_t *cseg, int G, int r, int
         base = __shfl(s, 63, 64);
     }
     return G - 1;  // unreachable when sum(cseg) covers every slot (validated on the host)
-}
-
-// The same search on inclusive prefix sums kept in LDS (entry g holds
-// cseg[0]+..+cseg[g]): no global memory access, so it can run while operand
-// loads are in flight without waiting for them.
-__device__ __forceinline__ int find_group_lds(const int *pre, int G, int r, int lane) {
-    for (int it = 0; it < G; it += 64) {
-        const int idx = it + lane;
-        unsigned long long hit = __ballot(idx < G && pre[idx] > r);
-        if (hit) return it + (int)__builtin_ctzll(hit);
-    }
-    return G - 1;
 }
 
 // s_waitcnt vmcnt(n) only (expcnt/lgkmcnt left at their maxima); gfx9 encoding:
@@ -139,31 +136,37 @@ __device__ __forceinline__ void dma_load16(const __attribute__((address_space(1)
 
 #define FO_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 
-template <typename Tag, int MTM, int MTN, int BK, int STAGES, int WM, int WN, int MODE>
+template <typename Tag, int MTM, int MTN, int BK, int SA, int SB, int WM, int WN, int MODE>
 __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
     typedef fo_elem<Tag> E;
     constexpr int NW = WM * WN;
     constexpr int CH = BK / 8;                  // 16-byte chunks per tile row
     constexpr int SWZ_SHIFT = CH == 8 ? 1 : 2;  // rows sharing one swizzle key: 16 / CH
     constexpr int WTM = MTM / WM, WTN = MTN / WN;
-    constexpr int FM = WTM / 32, FN = WTN / 32;
+    constexpr int FM = WTM / 16, FN = WTN / 16;  // 16x16 accumulator blocks per wavefront
+    constexpr int FMB = WTM / 32;                // 32-row groups of the epilogue
     constexpr int A_BLK = MTM * CH / 64, B_BLK = MTN * CH / 64;  // 1 KiB blocks per stage
     constexpr int PA = A_BLK / NW, PB = B_BLK / NW;              // blocks per wavefront
     constexpr int P = PA + PB;                                   // load instructions per wavefront and stage
+    constexpr int A16 = MTM * CH;                                // A part of a stage in 16-byte units
     constexpr int STAGE16 = (MTM + MTN) * CH;                    // stage size in 16-byte units
-    constexpr int KK = BK / 16;                                  // MFMA k-steps per stage
-    constexpr int NM = FM * FN, NR = FM + FN;
+    // LDS: stage-major, A part then B part; with SA = SB + 1 the last stage has an A part only
+    constexpr int RING16 = SB * STAGE16 + (SA - SB) * A16;
+    // vector memory instructions that may stay in flight when the next K step's operands are needed:
+    // everything requested after that step's last part (request order per step: B part, then A part)
+    constexpr int ALLOW = (SA - SB) * PA + (SB - 2) * P;
+    constexpr int KK = BK / 32;                                  // MFMA k-steps per stage
     // epilogue: per-wavefront strip of 32 rows x WTN columns in the ring behind slot 0
     constexpr int PITCH = WTN + 8;   // halfs; keeps 16-byte alignment, skews banks
     constexpr int CPR = WTN / 8;     // 16-byte chunks per strip row
     constexpr int RPP = 64 / CPR;    // strip rows per store pass
-    constexpr int NST = FM * (32 / RPP);  // store instructions per wavefront and tile
-    static_assert(BK == 32 || BK == 64, "BK");
+    constexpr int NST = FMB * (32 / RPP);  // store instructions per wavefront and tile
+    static_assert(BK == 64, "BK: two MFMA k-steps per stage (the B fragment buffers alternate with their parity)");
     static_assert(A_BLK % NW == 0 && B_BLK % NW == 0, "tile rows must split evenly over the wavefronts");
     static_assert((NW * (64 / CH)) % 32 == 0, "swizzle key must repeat across a wavefront's blocks");
-    static_assert(STAGES >= 2, "ring depth");
-    static_assert(NW * 32 * PITCH * 2 <= (STAGES - 1) * STAGE16 * 16, "the epilogue strips must fit behind ring slot 0");
-    static_assert((STAGES - 1) * P + NST < 64, "vmcnt range");
+    static_assert(SB >= 2 && (SA == SB || SA == SB + 1), "ring depths");
+    static_assert(NW * 32 * PITCH * 2 <= (RING16 - STAGE16) * 16, "the epilogue strips must fit behind stage 0");
+    static_assert(SA * PA + SB * PB + NST < 64, "vmcnt range");
 
     extern __shared__ fo_u32x4 smem[];
     const unsigned smem_lds = (unsigned)(uintptr_t)FO_LDS_PTR(smem);  // LDS byte address of the ring
@@ -180,12 +183,21 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
     const bool ktail = (p.K % BK) != 0;
     const int KT_full = ktail ? KT - 1 : KT;  // K steps whose loads need no special care
 
-    // Fragment addressing: lane l supplies row (l & 31), k-chunk (l >> 5) of
-    // each 32x16 operand block.
-    const int frow = lane & 31, fk = lane >> 5;
+    // Fragment addressing: lane l supplies row (l & 15), k-chunk (l >> 4) of
+    // each 16x32 operand block.
+    const int frow = lane & 15, fk = lane >> 4;
     const int fkey = (frow >> SWZ_SHIFT) & (CH - 1);
-    const int a_off = (wm * WTM + frow) * CH;
-    const int b_off = MTM * CH + (wn * WTN + frow) * CH;
+    // LDS byte addresses of this lane's 16 bytes in the first block of the A
+    // part / B part of stage 0 for MFMA k-step 0.  Everything else is derived
+    // from them inside a K step (slot: + multiple of the stage size, k-step:
+    // flip bit 2 of the chunk index, block: + immediate), from copies the compiler
+    // cannot see through: as loop invariants the derived addresses would occupy
+    // sixteen registers for the whole K loop.
+    const unsigned la = smem_lds + (unsigned)((wm * WTM + frow) * CH + (fk ^ fkey)) * 16;
+    const unsigned lb = smem_lds + (unsigned)(MTM * CH + (wn * WTN + frow) * CH + (fk ^ fkey)) * 16;
+    constexpr unsigned STAGE_B = STAGE16 * 16, BLOCK_B = 16 * CH * 16, KSTEP_X = 4 * 16;
+    static_assert(STAGE_B % (2 * KSTEP_X) == 0, "adding a slot offset must not disturb the k-step bit");
+    typedef const __attribute__((address_space(3))) fo_u32x4 *lds16_t;
 
     // Loader role of this lane inside a 1 KiB block: LDS slot `lane` is
     // (row lane / CH, physical chunk lane % CH); it must receive logical chunk
@@ -207,17 +219,34 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
         Ab = (gptr_t)(p.A) + ((size_t)pm_ * MTM + wave * (64 / CH)) * p.lda * 2;
         Bb = (gptr_t)(p.B) + ((size_t)pn_ * MTN + wave * (64 / CH)) * p.ldb * 2;
     };
-    // Issue the loads of K step kt into ring slot s (P instructions per wavefront).
-    auto issue_with = [&](int kt, int s, unsigned al, unsigned bl) {
-        const unsigned as = smem_lds + (unsigned)(s * STAGE16 + wave * 64) * 16;  // LDS byte addresses
-        const unsigned bs = as + MTM * CH * 16;
-        gptr_t ak = Ab + (size_t)kt * (BK * 2), bk = Bb + (size_t)kt * (BK * 2);
+    // Request the A part / B part of K step kt into slot s of its ring (PA / PB
+    // instructions per wavefront).
+    auto issue_a_with = [&](int kt, int s, unsigned al) {
+        const unsigned as = smem_lds + (unsigned)(s * STAGE16 + wave * 64) * 16;  // LDS byte address
+        gptr_t ak = Ab + (size_t)kt * (BK * 2);
 #pragma unroll
         for (int i = 0; i < PA; i++) dma_load16(ak + i * a_blk_bytes, al, as + i * NW * 1024);
+    };
+    auto issue_b_with = [&](int kt, int s, unsigned bl) {
+        const unsigned bs = smem_lds + (unsigned)(s * STAGE16 + A16 + wave * 64) * 16;
+        gptr_t bk = Bb + (size_t)kt * (BK * 2);
 #pragma unroll
         for (int i = 0; i < PB; i++) dma_load16(bk + i * b_blk_bytes, bl, bs + i * NW * 1024);
     };
-    auto issue = [&](int kt, int s) { issue_with(kt, s, a_lane, b_lane); };
+    auto issue_a = [&](int kt, int s) { issue_a_with(kt, s, a_lane); };
+    auto issue_b = [&](int kt, int s) { issue_b_with(kt, s, b_lane); };
+    // Load number q of the P a wavefront requests per K step (the B part of step
+    // kb into slot sb first, then the A part of step ka into slot sa), so that
+    // the steady loop can place them one by one between its MFMAs.
+    auto issue_one = [&](int q, int kb, int sb, int ka, int sa) {
+        if (q < PB) {
+            const unsigned bs = smem_lds + (unsigned)(sb * STAGE16 + A16 + wave * 64) * 16;
+            dma_load16(Bb + (size_t)kb * (BK * 2) + q * b_blk_bytes, b_lane, bs + q * NW * 1024);
+        } else {
+            const unsigned as = smem_lds + (unsigned)(sa * STAGE16 + wave * 64) * 16;
+            dma_load16(Ab + (size_t)ka * (BK * 2) + (q - PB) * a_blk_bytes, a_lane, as + (q - PB) * NW * 1024);
+        }
+    };
     // The partial last K step.  Whether this lane's chunk lies beyond K is
     // recomputed from a laundered lane id, so nothing of it stays live across
     // the K loop.
@@ -228,55 +257,91 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
         const int lc = (el % CH) ^ (((wave * (64 / CH) + el / CH) >> SWZ_SHIFT) & (CH - 1));
         return (KT - 1) * BK + lc * 8 >= p.K;
     };
-    // Same loads as issue(); a chunk beyond K is fetched from the row's first chunk of this step instead.
-    auto issue_any = [&](int kt, int s) {
+    // Same loads; in the partial step a chunk beyond K is fetched from the row's first chunk of that step instead.
+    auto issue_a_any = [&](int kt, int s) {
         if (ktail && kt == KT - 1) {
             int row;
             const bool out = tail_chunk_out(&row);
-            issue_with(kt, s, out ? (unsigned)(row * p.lda * 2) : a_lane, out ? (unsigned)(row * p.ldb * 2) : b_lane);
+            issue_a_with(kt, s, out ? (unsigned)(row * p.lda * 2) : a_lane);
         } else {
-            issue(kt, s);
+            issue_a(kt, s);
         }
     };
-    // Zero this lane's chunks of the partial step in ring slot s.  Called after
-    // the lane's own loads of that stage have landed and before the barrier that
-    // publishes the stage.
-    auto zero_tail = [&](int s) {
+    auto issue_b_any = [&](int kt, int s) {
+        if (ktail && kt == KT - 1) {
+            int row;
+            const bool out = tail_chunk_out(&row);
+            issue_b_with(kt, s, out ? (unsigned)(row * p.ldb * 2) : b_lane);
+        } else {
+            issue_b(kt, s);
+        }
+    };
+    // Zero this lane's chunks of the partial step (A part in slot sa, B part in
+    // slot sb).  Called after the lane's own loads of that step have landed and
+    // before the barrier that publishes it.
+    auto zero_tail = [&](int sa, int sb) {
         int row;
         if (tail_chunk_out(&row)) {
             int el = lane;
             asm volatile("" : "+v"(el));
-            fo_u32x4 *mine = smem + s * STAGE16 + wave * 64 + el;
+            fo_u32x4 *mine_a = smem + sa * STAGE16 + wave * 64 + el;
+            fo_u32x4 *mine_b = smem + sb * STAGE16 + A16 + wave * 64 + el;
             const fo_u32x4 z = {0u, 0u, 0u, 0u};
 #pragma unroll
-            for (int i = 0; i < PA; i++) mine[i * NW * 64] = z;
+            for (int i = 0; i < PA; i++) mine_a[i * NW * 64] = z;
 #pragma unroll
-            for (int i = 0; i < PB; i++) mine[MTM * CH + i * NW * 64] = z;
+            for (int i = 0; i < PB; i++) mine_b[i * NW * 64] = z;
         }
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    };
+    // Everything of a tile that is requested ahead of its first K step, except
+    // stage 0, in the order the K loop's waits assume: the A parts that run one
+    // step further ahead than the B parts first, then per step its B part and
+    // the A part requested with it.
+    auto issue_rest_of_prologue = [&]() {
+#pragma unroll
+        for (int k = 1; k <= SA - SB; k++)
+            if (k < KT) issue_a_any(k, k);
+#pragma unroll
+        for (int k = 1; k < SB; k++) {
+            if (k < KT) issue_b_any(k, k);
+            if (k + SA - SB < KT) issue_a_any(k + SA - SB, k + SA - SB);
+        }
     };
 
     // ---- signalling state (signal and scatter epilogues)
     const int sub_n = MTN / p.BN, nsub = (MTM / p.BM) * sub_n;  // reorder tiles per macro tile
     typedef const __attribute__((address_space(4))) int32_t *cptr_t;  // read-only for the whole launch: scalar loads
     const cptr_t RAc = (cptr_t)(uintptr_t)p.RA;
-    int *pre = reinterpret_cast<int *>(smem + STAGES * STAGE16);  // behind the ring: prefix sums of cseg
-    const bool lds_search = p.G <= kPrefixMax;
-    if (MODE != MODE_PLAIN && wave == 0 && lds_search) {
-        int base = 0;
-        for (int it = 0; it < p.G; it += 64) {
-            const int idx = it + lane;
-            int s = idx < p.G ? p.cseg[idx] : 0;
+    // Inclusive prefix sums of cseg, entries lane and lane + 64, in two registers
+    // of every lane (the search below is a ballot over them: no memory access, so
+    // it can run while operand loads are in flight without waiting for them).
+    // More than kPrefixRegs groups are searched in memory.
+    int pre0 = 0, pre1 = 0;
+    const bool reg_search = p.G <= kPrefixRegs;
+    if (MODE != MODE_PLAIN && reg_search) {
+        int s0 = lane < p.G ? p.cseg[lane] : 0;
+        int s1 = lane + 64 < p.G ? p.cseg[lane + 64] : 0;
 #pragma unroll
-            for (int d = 1; d < 64; d <<= 1) {
-                int o = __shfl_up(s, d, 64);
-                if (lane >= d) s += o;
+        for (int d = 1; d < 64; d <<= 1) {
+            int o0 = __shfl_up(s0, d, 64), o1 = __shfl_up(s1, d, 64);
+            if (lane >= d) {
+                s0 += o0;
+                s1 += o1;
             }
-            s += base;
-            if (idx < p.G) pre[idx] = s;  // read back by wavefront 0 only, after later barriers
-            base = __shfl(s, 63, 64);
         }
+        pre0 = s0;
+        pre1 = s1 + __shfl(s0, 63, 64);
     }
+    auto group_of = [&](int r) {
+        if (reg_search) {
+            unsigned long long hit = __ballot(lane < p.G && pre0 > r);
+            if (hit) return (int)__builtin_ctzll(hit);
+            hit = __ballot(lane + 64 < p.G && pre1 > r);
+            return hit ? 64 + (int)__builtin_ctzll(hit) : p.G - 1;
+        }
+        return find_group(p.cseg, p.G, r, lane);
+    };
     // Wavefront 0 announces the reorder tiles whose storage slots are rs[0..nsub).
     // Callers guarantee that every wavefront's stores of those tiles are complete:
     // the stores are write-through, each wavefront has waited for their
@@ -290,7 +355,7 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
         for (int s = 0; s < kMaxSub; s++) {
             if (s < nsub) {
                 const int r = rs[s];
-                const int g = lds_search ? find_group_lds(pre, p.G, r, lane) : find_group(p.cseg, p.G, r, lane);
+                const int g = group_of(r);
                 if (lane == 0) {
                     __hip_atomic_fetch_add(p.MM + g, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     if (p.monitor) {
@@ -303,82 +368,98 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
         }
     };
 
-    // Operand fragments are double buffered in registers: while the MFMAs of
-    // k-step kk run, the ds_reads of k-step kk+1 (or of the next stage's first
-    // k-step) are in flight.
-    fo_float16v acc[FM][FN];
-    fo_u32x4 af[2][FM], bf[2][FN];
-#define FO_LOAD_FRAGS(buf_, st_, kk_)                                                                 \
-    {                                                                                                 \
-        const int c_ = ((kk_) * 2 + fk) ^ fkey;                                                       \
-        _Pragma("unroll") for (int i = 0; i < FM; i++) af[buf_][i] = (st_)[a_off + i * 32 * CH + c_]; \
-        _Pragma("unroll") for (int j = 0; j < FN; j++) bf[buf_][j] = (st_)[b_off + j * 32 * CH + c_]; \
-    }
-    // The N-side block is the MFMA's first operand, so a lane's four consecutive
-    // accumulator values are consecutive output columns.
-#define FO_MFMAS(kk_)                                  \
-    _Pragma("unroll") for (int i = 0; i < FM; i++)     \
-        _Pragma("unroll") for (int j = 0; j < FN; j++) \
-            acc[i][j] = E::mfma(bf[(kk_) & 1][j], af[(kk_) & 1][i], acc[i][j]);
+    // Operand fragments.  A K step is walked as KK * FM "rows": the FN MFMAs of
+    // one A fragment (16 rows of A, 32 columns of K).  An A fragment is dead after
+    // its row, so the A side is a short ring: the fragment of row r + AHEAD is
+    // fetched right behind row r into the registers row r - 1 used.  The B
+    // fragments of an MFMA k-step are live for its FM rows; the next k-step's are
+    // fetched during its last FN rows into a second set.
+    constexpr int AHEAD = 3, ARING = AHEAD + 1;
+    constexpr int ROWS = KK * FM;
+    static_assert(FM % ARING == 0 && FN <= FM && AHEAD < FM, "row pipeline");
+    fo_float4v acc[FM][FN];
+    fo_u32x4 af[ARING], bf[2][FN];
+    // base = la or lb (or a laundered copy) + slot * STAGE_B
+    auto load_a = [&](int slot, unsigned base, int kk, int i) {
+        af[slot] = *reinterpret_cast<lds16_t>((base ^ (kk * KSTEP_X)) + i * BLOCK_B);
+    };
+    auto load_b = [&](int buf, unsigned base, int kk, int j) {
+        bf[buf][j] = *reinterpret_cast<lds16_t>((base ^ (kk * KSTEP_X)) + j * BLOCK_B);
+    };
 
     int prev_rs[kMaxSub] = {0, 0, 0, 0};  // slots of the tile whose signal is still owed
     bool owed = false;
 
-    // One K step.  STEADY: at least STAGES further steps exist, so the waits and
-    // the refill are unconditional and the body is a single scheduling region
-    // per k-step, pinned MFMA-first with the memory instructions in its shadow.
-    // With two slots the steady loop is unrolled by two and the slot is a
-    // compile-time constant (slot_tag >= 0), which makes every LDS address
+    // One K step kt, whose A part is in slot sa of the A ring and whose B part is
+    // in slot sb of the B ring.  STEADY: at least SA further full steps exist, so
+    // the waits and the refill are unconditional and the body is a single
+    // scheduling region per k-step, pinned MFMA-first with the memory
+    // instructions in its shadow.  In the unrolled steady loops the slots are
+    // compile-time constants (tags >= 0), which makes every LDS address
     // loop-invariant.  `first` marks a tile's first K step: after its barrier
     // every wavefront has waited for the previous tile's stores (they are older
     // than the loads that wait covers), which is where an owed signal is sent.
-    auto kstep = [&](auto steady, auto slot_tag, bool first, int kt, int slot_rt, int nslot_rt) {
+    auto kstep = [&](auto steady, auto tag_a, auto tag_b, bool first, int kt, int sa_rt, int sb_rt) {
         constexpr bool STEADY = decltype(steady)::value;
-        constexpr int SLOT_C = decltype(slot_tag)::value;
-        const int slot = SLOT_C >= 0 ? SLOT_C : slot_rt;
-        const int nslot = SLOT_C >= 0 ? (SLOT_C ^ 1) : nslot_rt;
-        const fo_u32x4 *st = smem + slot * STAGE16;
+        constexpr int SA_C = decltype(tag_a)::value, SB_C = decltype(tag_b)::value;
+        const int sa = SA_C >= 0 ? SA_C : sa_rt;
+        const int sb = SB_C >= 0 ? SB_C : sb_rt;
+        const int nsa = sa + 1 == SA ? 0 : sa + 1;
+        const int nsb = sb + 1 == SB ? 0 : sb + 1;
+        unsigned la_ = la, lb_ = lb;
+        asm volatile("" : "+v"(la_), "+v"(lb_));
+        const unsigned sta = la_ + sa * STAGE_B, stb = lb_ + sb * STAGE_B;
+        const unsigned nsta = la_ + nsa * STAGE_B, nstb = lb_ + nsb * STAGE_B;
+        const bool more = STEADY || kt + 1 < KT;  // a further K step follows in this tile
+        // Row SYNC is the last whose fetches read step kt (the A fragment of the
+        // step's last row; the last B fragments were fetched in the k-step
+        // before).  Behind them the workgroup meets: every wavefront has issued
+        // its last reads of step kt, so the two slots can be recycled, and step
+        // kt+1 is made visible (own loads landed + barrier) for the fetches of
+        // the remaining rows, which already belong to it.
+        constexpr int SYNC = ROWS - 1 - AHEAD;
+        static_assert(FN <= AHEAD + 1 && SYNC >= ROWS - FM, "the rows behind SYNC fetch the next step's first B fragments");
 #pragma unroll
-        for (int kk = 0; kk < KK; kk++) {
-            if (kk + 1 < KK) {
-                FO_LOAD_FRAGS((kk + 1) & 1, st, kk + 1)
-            } else if (STEADY || kt + 1 < KT) {
-                // This wavefront holds all of stage kt in registers.  Make stage
-                // kt+1 visible (own loads landed + barrier), then recycle slot kt
-                // for stage kt+STAGES and fetch the next stage's first fragments.
-                if (STEADY || kt + STAGES - 1 < KT)
-                    wait_vmcnt<(STAGES - 2) * P>();
-                else
-                    wait_vmcnt<0>();
-                if (!STEADY) {
-                    if (ktail && kt + 2 == KT) zero_tail(nslot);  // all loads of stage KT-1 have landed (vmcnt 0)
-                }
-                __builtin_amdgcn_s_barrier();
-                asm volatile("" ::: "memory");
-                if (!STEADY && MODE != MODE_PLAIN) {
-                    if (first && owed && wave == 0) announce(prev_rs);
-                }
-                if constexpr (STEADY) {
-                    issue(kt + STAGES, slot);
-                } else {
-                    if (kt + STAGES < KT) issue_any(kt + STAGES, slot);
-                }
-                FO_LOAD_FRAGS((kk + 1) & 1, smem + nslot * STAGE16, 0)
-            }
-            FO_MFMAS(kk)
-            if (STEADY) {
-                // issue order inside this k-step: MFMA, ds_read, MFMA, ds_read, ...
-                // then (last k-step) the direct-to-LDS loads between the remaining MFMAs
+        for (int r = 0; r < ROWS; r++) {
+            const int kk = r / FM, i = r % FM;
+            const bool last = kk + 1 == KK;
+            // One row is one scheduling region: its FN MFMAs, the A fragment of
+            // row r + AHEAD, one B fragment of the next k-step in the rows that
+            // fetch those, and behind SYNC a share of the direct-to-LDS loads.
+            // Nothing may move across a row: a fetch hoisted above the MFMAs that
+            // still read the registers it replaces would cost a second register set.
 #pragma unroll
-                for (int t = 0; t < NM; t++) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    if (t < NR) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                    if (kk + 1 == KK) {
-                        constexpr int per = (P + NM - 1) / NM;
-                        __builtin_amdgcn_sched_group_barrier(0x010, per, 0);
+            for (int j = 0; j < FN; j++) E::mfma(bf[kk & 1][j], af[r % ARING], acc[i][j]);
+            if (r + AHEAD < ROWS) load_a((r + AHEAD) % ARING, sta, (r + AHEAD) / FM, (r + AHEAD) % FM);
+            if (!last && i >= FM - FN) load_b((kk + 1) & 1, stb, kk + 1, i - (FM - FN));
+            if (r >= SYNC && more) {
+                if (r == SYNC) {
+                    if (STEADY || kt + SA - 1 < KT)
+                        wait_vmcnt<ALLOW>();
+                    else
+                        wait_vmcnt<0>();
+                    if (!STEADY) {
+                        if (ktail && kt + 2 == KT) zero_tail(nsa, nsb);  // all loads of step KT-1 have landed (vmcnt 0)
+                    }
+                    __builtin_amdgcn_s_barrier();
+                    asm volatile("" ::: "memory");
+                    if (!STEADY && MODE != MODE_PLAIN) {
+                        if (first && owed && wave == 0) announce(prev_rs);
+                    }
+                    if constexpr (!STEADY) {
+                        if (kt + SB < KT) issue_b_any(kt + SB, sb);
+                        if (kt + SA < KT) issue_a_any(kt + SA, sa);
                     }
                 }
+                if (r > SYNC) load_a((r + AHEAD) % ARING, nsta, 0, r + AHEAD - ROWS);
+                if (r - SYNC < FN) load_b(KK & 1, nstb, 0, r - SYNC);
+                if constexpr (STEADY) {
+#pragma unroll
+                    for (int q = (r - SYNC) * P / (AHEAD + 1); q < (r - SYNC + 1) * P / (AHEAD + 1); q++)
+                        issue_one(q, kt + SB, sb, kt + SA, sa);
+                }
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
@@ -389,7 +470,8 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
     pm = __builtin_amdgcn_readfirstlane(pm);
     pn = __builtin_amdgcn_readfirstlane(pn);
     set_tile(pm, pn);
-    issue_any(0, 0);
+    issue_a_any(0, 0);
+    issue_b_any(0, 0);
     bool carried = false;  // stores of an earlier tile may still be in flight
 
     for (;;) {
@@ -405,63 +487,81 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
 #pragma unroll
             for (int j = 0; j < FN; j++)
 #pragma unroll
-                for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+                for (int v = 0; v < 4; v++) acc[i][j][v] = 0.f;
+        fo_mfma_fence();
 
         // Stage 0 of this tile is in flight.  First tile: request the rest of the
-        // ring, then wait for stage 0.  Later tiles: stage 0 was requested before
-        // the previous epilogue, whose strips lived behind slot 0, so the rest
-        // of the ring is requested only after the barrier; the previous tile's
-        // NST stores are younger than stage 0 and need not have completed.
+        // prologue, then wait for stage 0.  Later tiles: stage 0 was requested
+        // before the previous epilogue, whose strips lived behind stage 0, so the
+        // rest is requested only after the barrier; the previous tile's NST
+        // stores are younger than stage 0 and need not have completed.
         if (!carried) {
-#pragma unroll
-            for (int s = 1; s < STAGES; s++)
-                if (s < KT) issue_any(s, s);
-            if (KT >= STAGES)
-                wait_vmcnt<(STAGES - 1) * P>();
+            issue_rest_of_prologue();
+            if (KT >= SA)
+                wait_vmcnt<(SA - 1) * PA + (SB - 1) * PB>();
             else
                 wait_vmcnt<0>();
-            if (ktail && KT == 1) zero_tail(0);
+            if (ktail && KT == 1) zero_tail(0, 0);
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
         } else {
             wait_vmcnt<NST>();
-            if (ktail && KT == 1) zero_tail(0);
+            if (ktail && KT == 1) zero_tail(0, 0);
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-#pragma unroll
-            for (int s = 1; s < STAGES; s++)
-                if (s < KT) issue_any(s, s);
+            issue_rest_of_prologue();
         }
-        FO_LOAD_FRAGS(0, smem, 0)
+#pragma unroll
+        for (int j = 0; j < FN; j++) load_b(0, lb, 0, j);
+#pragma unroll
+        for (int i = 0; i < AHEAD; i++) load_a(i, la, 0, i);
 
         using dyn = std::integral_constant<int, -1>;
-        int slot = 0;  // ring slot of K step kt
+        using yes = std::true_type;
+        using no = std::false_type;
+#define FO_SLOT(n_) std::integral_constant<int, (n_)>{}
+        int sa = 0, sb = 0;  // ring slots of K step kt
         int kt = 0;
-        for (; kt < STAGES - 1 && kt < KT; kt++) {
-            const int nslot = slot + 1 == STAGES ? 0 : slot + 1;
-            kstep(std::false_type{}, dyn{}, kt == 0, kt, slot, nslot);
-            slot = nslot;
+        auto advance = [&]() {
+            sa = sa + 1 == SA ? 0 : sa + 1;
+            sb = sb + 1 == SB ? 0 : sb + 1;
+            kt++;
+        };
+        // the first step is never a steady one: it may carry the previous tile's signal
+        if (kt < KT) {
+            kstep(no{}, dyn{}, dyn{}, true, kt, sa, sb);
+            advance();
         }
         if (MODE != MODE_PLAIN && KT >= 2) owed = false;  // sent in the first K step
-        if constexpr (STAGES == 2) {
-            // here kt == 1 (slot 1) when KT > 1
-            for (; kt + 1 + STAGES < KT_full; kt += 2) {
-                kstep(std::true_type{}, std::integral_constant<int, 1>{}, false, kt, 1, 0);
-                kstep(std::true_type{}, std::integral_constant<int, 0>{}, false, kt + 1, 0, 1);
+        // steady loops start at kt == 1, slots 1 and 1
+        if constexpr (SA == 2 && SB == 2) {
+            for (; kt + 1 + SA < KT_full; kt += 2) {
+                kstep(yes{}, FO_SLOT(1), FO_SLOT(1), false, kt, 1, 1);
+                kstep(yes{}, FO_SLOT(0), FO_SLOT(0), false, kt + 1, 0, 0);
+            }
+        } else if constexpr (SA == 3 && SB == 2) {
+            for (; kt + 5 + SA < KT_full; kt += 6) {
+                kstep(yes{}, FO_SLOT(1), FO_SLOT(1), false, kt, 1, 1);
+                kstep(yes{}, FO_SLOT(2), FO_SLOT(0), false, kt + 1, 2, 0);
+                kstep(yes{}, FO_SLOT(0), FO_SLOT(1), false, kt + 2, 0, 1);
+                kstep(yes{}, FO_SLOT(1), FO_SLOT(0), false, kt + 3, 1, 0);
+                kstep(yes{}, FO_SLOT(2), FO_SLOT(1), false, kt + 4, 2, 1);
+                kstep(yes{}, FO_SLOT(0), FO_SLOT(0), false, kt + 5, 0, 0);
             }
         } else {
-            for (; kt + STAGES < KT_full; kt++) {
-                const int nslot = slot + 1 == STAGES ? 0 : slot + 1;
-                kstep(std::true_type{}, dyn{}, false, kt, slot, nslot);
-                slot = nslot;
+            for (; kt + SA < KT_full;) {
+                kstep(yes{}, dyn{}, dyn{}, false, kt, sa, sb);
+                advance();
             }
         }
-        for (; kt < KT; kt++) {
-            const int nslot = slot + 1 == STAGES ? 0 : slot + 1;
-            kstep(std::false_type{}, dyn{}, kt == 0, kt, slot, nslot);
-            slot = nslot;
+        while (kt < KT) {
+            kstep(no{}, dyn{}, dyn{}, false, kt, sa, sb);
+            advance();
         }
+#undef FO_SLOT
 
+
+        fo_mfma_fence();
         // every wavefront is done reading the ring (no loads are in flight here)
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
         __builtin_amdgcn_s_barrier();
@@ -476,7 +576,8 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
             pm = __builtin_amdgcn_readfirstlane(pm);
             pn = __builtin_amdgcn_readfirstlane(pn);
             set_tile(pm, pn);
-            issue_any(0, 0);
+            issue_a_any(0, 0);
+            issue_b_any(0, 0);
         }
 
         // ---- epilogue: accumulators -> 16-bit -> LDS (per-wave strip of 32 rows) -> global
@@ -488,7 +589,7 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
         {
             int el = lane;
             asm volatile("" : "+v"(el));
-            const int erow = el & 31, ek = el >> 5;
+            const int erow = el & 15, ek = el >> 4;  // accumulator block: row erow, columns 4*ek .. 4*ek+3
             uint16_t *strip = reinterpret_cast<uint16_t *>(smem + STAGE16) + wave * (32 * PITCH);
             const int srow = el / CPR, scol = el % CPR;
             const int ldp = MODE == MODE_PLAIN ? p.N : p.rLDN * p.BN;  // leading dimension of the output view
@@ -505,28 +606,29 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
             char *cbase = reinterpret_cast<char *>(p.C) + (trow * ldp + tcol) * 2;  // wave-uniform
             const unsigned lane_off = (unsigned)(srow * ldp + scol * 8) * 2;
             // scatter: the row map entries of all rows this lane will store, fetched in one batch
-            int32_t dest_row[MODE == MODE_SCATTER ? FM * (32 / RPP) : 1];
+            int32_t dest_row[MODE == MODE_SCATTER ? FMB * (32 / RPP) : 1];
             if (MODE == MODE_SCATTER) {
 #pragma unroll
-                for (int i = 0; i < FM; i++)
+                for (int i = 0; i < FMB; i++)
 #pragma unroll
                     for (int ps = 0; ps < 32 / RPP; ps++)
                         dest_row[i * (32 / RPP) + ps] = p.RE[trow + i * 32 + ps * RPP + srow];
             }
 #pragma unroll
-            for (int i = 0; i < FM; i++) {
+            for (int i = 0; i < FMB; i++) {  // 32 output rows = two rows of accumulator blocks
 #pragma unroll
-                for (int j = 0; j < FN; j++) {
+                for (int ii = 0; ii < 2; ii++) {
 #pragma unroll
-                    for (int q = 0; q < 4; q++) {
-                        uint16_t h0 = E::from_f32(acc[i][j][q * 4 + 0]);
-                        uint16_t h1 = E::from_f32(acc[i][j][q * 4 + 1]);
-                        uint16_t h2 = E::from_f32(acc[i][j][q * 4 + 2]);
-                        uint16_t h3 = E::from_f32(acc[i][j][q * 4 + 3]);
+                    for (int j = 0; j < FN; j++) {
+                        const fo_float4v a4 = acc[i * 2 + ii][j];
+                        uint16_t h0 = E::from_f32(a4[0]);
+                        uint16_t h1 = E::from_f32(a4[1]);
+                        uint16_t h2 = E::from_f32(a4[2]);
+                        uint16_t h3 = E::from_f32(a4[3]);
                         fo_u32x2 v;
                         v.x = (uint32_t)h0 | ((uint32_t)h1 << 16);
                         v.y = (uint32_t)h2 | ((uint32_t)h3 << 16);
-                        *reinterpret_cast<fo_u32x2 *>(strip + erow * PITCH + j * 32 + q * 8 + ek * 4) = v;
+                        *reinterpret_cast<fo_u32x2 *>(strip + (ii * 16 + erow) * PITCH + j * 16 + ek * 4) = v;
                     }
                 }
                 // the strip is private to this wavefront: order its LDS writes before its reads
@@ -575,15 +677,13 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
         carried = true;
         tile = next;
     }
-#undef FO_LOAD_FRAGS
-#undef FO_MFMAS
 }
 
-// Dynamic LDS of one workgroup: the ring (the epilogue strips reuse its last
-// slot) and the table of group prefix sums.
-template <int MTM, int MTN, int BK, int STAGES>
+// Dynamic LDS of one workgroup: the two rings (the epilogue strips reuse the
+// space behind stage 0).
+template <int MTM, int MTN, int BK, int SA, int SB>
 constexpr int smem_bytes() {
-    return STAGES * (MTM + MTN) * BK * 2 + kPrefixMax * 4;
+    return (SB * (MTM + MTN) + (SA - SB) * MTM) * BK * 2;
 }
 
 }  // namespace fo_gemm_dev
