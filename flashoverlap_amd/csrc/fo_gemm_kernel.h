@@ -375,6 +375,10 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
     // fragments of an MFMA k-step are live for its FM rows; the next k-step's are
     // fetched during its last FN rows into a second set.
     constexpr int AHEAD = 3, ARING = AHEAD + 1;
+    // The step's P direct-to-LDS loads are dealt over the rows behind its barrier
+    // instead of being issued in one burst (measured: 3 % faster; AHEAD = 7 with
+    // the loads over eight rows another 0.7 %, for 16 more registers).
+    constexpr int DMA_ROWS = AHEAD + 1;
     constexpr int ROWS = KK * FM;
     static_assert(FM % ARING == 0 && FN <= FM && AHEAD < FM, "row pipeline");
     fo_float4v acc[FM][FN];
@@ -455,8 +459,8 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
                 if (r - SYNC < FN) load_b(KK & 1, nstb, 0, r - SYNC);
                 if constexpr (STEADY) {
 #pragma unroll
-                    for (int q = (r - SYNC) * P / (AHEAD + 1); q < (r - SYNC + 1) * P / (AHEAD + 1); q++)
-                        issue_one(q, kt + SB, sb, kt + SA, sa);
+                    for (int q = 0; q < P; q++)
+                        if (q * DMA_ROWS / P == r - SYNC) issue_one(q, kt + SB, sb, kt + SA, sa);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
