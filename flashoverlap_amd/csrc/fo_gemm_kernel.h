@@ -342,20 +342,26 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
         }
         return find_group(p.cseg, p.G, r, lane);
     };
-    // Wavefront 0 announces the reorder tiles whose storage slots are rs[0..nsub).
-    // Callers guarantee that every wavefront's stores of those tiles are complete:
+    // Wavefront 0 announces the reorder tiles whose storage slots are rs[0..nsub)
+    // and whose groups are gs[0..nsub).  (The groups are looked up by the caller,
+    // at the end of the epilogue: the lookup inside a K step measured 3 us per
+    // tile, the counter update alone nothing.)  Callers guarantee that every wavefront's stores of those tiles are complete:
     // the stores are write-through, each wavefront has waited for their
     // acknowledgement (vmcnt) and a workgroup barrier lies between that wait and
     // this call.  The tile is therefore in memory before the counter moves, and
     // the atomic itself is relaxed: a release here would add an L2 write-back
     // (with nothing of this tile left to write back) and a wait for the operand
     // loads in flight, both paid by the whole workgroup at its next barrier.
-    auto announce = [&](const int (&rs)[kMaxSub]) {
+    auto groups_of = [&](const int (&rs)[kMaxSub], int (&gs)[kMaxSub]) {
+#pragma unroll
+        for (int s = 0; s < kMaxSub; s++) gs[s] = s < nsub ? group_of(rs[s]) : 0;
+    };
+    auto announce = [&](const int (&rs)[kMaxSub], const int (&gs)[kMaxSub]) {
 #pragma unroll
         for (int s = 0; s < kMaxSub; s++) {
             if (s < nsub) {
                 const int r = rs[s];
-                const int g = group_of(r);
+                const int g = gs[s];
                 if (lane == 0) {
                     __hip_atomic_fetch_add(p.MM + g, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     if (p.monitor) {
@@ -391,7 +397,8 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
         bf[buf][j] = *reinterpret_cast<lds16_t>((base ^ (kk * KSTEP_X)) + j * BLOCK_B);
     };
 
-    int prev_rs[kMaxSub] = {0, 0, 0, 0};  // slots of the tile whose signal is still owed
+    int prev_rs[kMaxSub] = {0, 0, 0, 0};  // slots and groups of the tile whose signal is still owed
+    int prev_gs[kMaxSub] = {0, 0, 0, 0};
     bool owed = false;
 
     // One K step kt, whose A part is in slot sa of the A ring and whose B part is
@@ -448,7 +455,7 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
                     __builtin_amdgcn_s_barrier();
                     asm volatile("" ::: "memory");
                     if (!STEADY && MODE != MODE_PLAIN) {
-                        if (first && owed && wave == 0) announce(prev_rs);
+                        if (first && owed && wave == 0) announce(prev_rs, prev_gs);
                     }
                     if constexpr (!STEADY) {
                         if (kt + SB < KT) issue_b_any(kt + SB, sb);
@@ -661,11 +668,16 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
         }
 
         if (MODE != MODE_PLAIN) {
+            int gs[kMaxSub] = {0, 0, 0, 0};
+            if (wave == 0) groups_of(rs, gs);
             if (has_next && KT >= 2) {
                 // sent from inside the next tile's first K step
                 owed = true;
 #pragma unroll
-                for (int s = 0; s < kMaxSub; s++) prev_rs[s] = rs[s];
+                for (int s = 0; s < kMaxSub; s++) {
+                    prev_rs[s] = rs[s];
+                    prev_gs[s] = gs[s];
+                }
             } else {
                 // Every lane waits until its own stores are acknowledged, the
                 // barrier collects the workgroup, and only then one lane
@@ -674,7 +686,7 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
                 __builtin_amdgcn_s_waitcnt(0);
                 __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
-                if (wave == 0) announce(rs);
+                if (wave == 0) announce(rs, gs);
             }
         }
         if (!has_next) break;
