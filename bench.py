@@ -278,7 +278,9 @@ def main():
         "dtype": dt, "data": "synthetic",
         "config": {"workload": f"{args.workload}: {desc}", "M": M, "N": N, "K": K, "tile": [BM, BN],
                    "groups": len(cseg), "cseg": cseg if len(cseg) <= 16 else f"{len(cseg)} x {cseg[0]}", "algo": algo,
-                   "consumer_launches": "one wait and one consumer launch per GEMM wave" if (args.fused == 0 or (args.fused < 0 and len(cseg) <= 16))
+                   "consumer_launches": "on the GEMM stream behind the GEMM (automatic choice for a GEMM this short)"
+                   if (args.fused < 0 and 2.0 * M * N * K < 6.4e10)
+                   else "one wait and one consumer launch per GEMM wave" if (args.fused == 0 or (args.fused < 0 and len(cseg) <= 16))
                    else "one"},
         "roofline": {"bound": "mfma", "kernel": "fo_gemm_kernel (signal epilogue)",
                      "achieved": achieved, "peak": PEAK_TFLOPS, "unit": "TFLOP/s",

@@ -34,9 +34,12 @@ __global__ void fo_set_kernel(int32_t *word, int value) {
     __hip_atomic_store(word, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// The same for `count` consecutive groups, one after the other.
-__global__ void fo_wait_groups_kernel(int count, const int32_t *expect, int32_t *counters, long max_polls) {
-    for (int g = 0; g < count; g++) {
+// The same for `count` consecutive groups: one wavefront, lane l takes groups
+// l, l + 64, ...  (a single lane walking 256 counters one after the other
+// measured 130 us on counters that were all complete already).
+__global__ __launch_bounds__(64) void fo_wait_groups_kernel(int count, const int32_t *expect, int32_t *counters,
+                                                            long max_polls) {
+    for (int g = threadIdx.x; g < count; g += 64) {
         const int want = expect[g];
         long polls = 0;
         for (;;) {
@@ -393,8 +396,8 @@ extern "C" int fo_set(int32_t *word, int value, fo_stream_t stream) {
 
 extern "C" int fo_wait_groups(int count, const int32_t *expect_dev, int32_t *counters, fo_stream_t stream) {
     if (count <= 0 || !expect_dev || !counters) return FO_ERR_ARG;
-    hipLaunchKernelGGL(fo_wait_groups_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream), count,
-                       expect_dev, counters, default_max_polls());
+    hipLaunchKernelGGL(fo_wait_groups_kernel, dim3(1), dim3(count < 64 ? count : 64), 0,
+                       static_cast<hipStream_t>(stream), count, expect_dev, counters, default_max_polls());
     FO_LAUNCH_CHECK();
     return FO_OK;
 }

@@ -62,7 +62,7 @@ struct GemmArgs {
 };
 
 constexpr int kMaxSub = 4;        // reorder tiles per macro tile (256x256 over 128x128)
-constexpr int kPrefixRegs = 128;  // group search on prefix sums held in two registers per lane up to this many groups
+constexpr int kPrefixRegs = 256;  // group search on prefix sums held in registers (one per 64 groups) up to this many groups
 
 // Group of storage slot r: smallest g with cseg[0]+..+cseg[g] > r
 // (src/overlap/gemm_with_signal.h:343-349), found by one wavefront with a
@@ -313,32 +313,37 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
     const int sub_n = MTN / p.BN, nsub = (MTM / p.BM) * sub_n;  // reorder tiles per macro tile
     typedef const __attribute__((address_space(4))) int32_t *cptr_t;  // read-only for the whole launch: scalar loads
     const cptr_t RAc = (cptr_t)(uintptr_t)p.RA;
-    // Inclusive prefix sums of cseg, entries lane and lane + 64, in two registers
-    // of every lane (the search below is a ballot over them: no memory access, so
-    // it can run while operand loads are in flight without waiting for them).
-    // More than kPrefixRegs groups are searched in memory.
-    int pre0 = 0, pre1 = 0;
+    // Inclusive prefix sums of cseg, entries lane, lane + 64, ... in kPrefixRegs / 64
+    // registers of every lane (the search below is a ballot over them: no memory
+    // access, so it never waits behind operand loads in flight).  More than
+    // kPrefixRegs groups are searched in memory.
+    constexpr int NPRE = kPrefixRegs / 64;
+    int pre[NPRE];
+#pragma unroll
+    for (int q = 0; q < NPRE; q++) pre[q] = 0;
     const bool reg_search = p.G <= kPrefixRegs;
     if (MODE != MODE_PLAIN && reg_search) {
-        int s0 = lane < p.G ? p.cseg[lane] : 0;
-        int s1 = lane + 64 < p.G ? p.cseg[lane + 64] : 0;
+        int base = 0;
 #pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            int o0 = __shfl_up(s0, d, 64), o1 = __shfl_up(s1, d, 64);
-            if (lane >= d) {
-                s0 += o0;
-                s1 += o1;
+        for (int q = 0; q < NPRE; q++) {
+            int v = q * 64 + lane < p.G ? p.cseg[q * 64 + lane] : 0;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                int o = __shfl_up(v, d, 64);
+                if (lane >= d) v += o;
             }
+            pre[q] = v + base;
+            base = __shfl(pre[q], 63, 64);
         }
-        pre0 = s0;
-        pre1 = s1 + __shfl(s0, 63, 64);
     }
     auto group_of = [&](int r) {
         if (reg_search) {
-            unsigned long long hit = __ballot(lane < p.G && pre0 > r);
-            if (hit) return (int)__builtin_ctzll(hit);
-            hit = __ballot(lane + 64 < p.G && pre1 > r);
-            return hit ? 64 + (int)__builtin_ctzll(hit) : p.G - 1;
+#pragma unroll
+            for (int q = 0; q < NPRE; q++) {
+                unsigned long long hit = __ballot(q * 64 + lane < p.G && pre[q] > r);
+                if (hit) return q * 64 + (int)__builtin_ctzll(hit);
+            }
+            return p.G - 1;
         }
         return find_group(p.cseg, p.G, r, lane);
     };

@@ -26,6 +26,17 @@ namespace {
 // needs no polling workgroups resident beside the GEMM.
 constexpr int kFusedFromGroups = 16;
 
+// In automatic mode a GEMM shorter than this many flop (about 50 us of this
+// GPU) keeps the whole call on the GEMM stream: signal GEMM, one wait that
+// resets every counter, one consumer launch.  Fork, join and pollers beside the
+// GEMM cost more than such a GEMM can hide (4096x4096x512 with 256 groups:
+// 71 us overlapped, 48 us in stream).
+constexpr double kInStreamBelowFlop = 6.4e10;
+
+bool in_stream(const fo_overlap *h, int M, int N, int K) {
+    return h->fused < 0 && 2.0 * M * N * K < kInStreamBelowFlop;
+}
+
 int fused_grid(const fo_overlap *h, int G) {  // 0: per-group launches, otherwise workgroups of the one launch
     if (h->fused < 0) return G > kFusedFromGroups ? 256 : 0;
     if (h->fused == 1) return 256;
@@ -235,15 +246,21 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
     const int64_t tile_elems = (int64_t)info[0] * info[1];
     if (h->acc && h->acc_nelem < (int64_t)M * N) return FO_ERR_ARG;
 
-    const int fused = fused_grid(h, G);
+    const bool same_stream = in_stream(h, M, N, K);
+    const int fused = same_stream ? 0 : fused_grid(h, G);
+    fo_stream_t cstream = same_stream ? h->gemm_stream : h->comm_stream;
     int32_t wave = 0;
-    if (!fused) {
+    if (same_stream) {
+        wave = TM * TN;  // every group in one batch
+    } else if (!fused) {
         rc = fo_gemm_wave_tiles(dtype, algo, M, N, &wave);
         if (rc) return rc;
     }
     const bool captured = capturing(h);
-    rc = fork(h, captured, fused != 0);
-    if (rc) return rc;
+    if (!same_stream) {
+        rc = fork(h, captured, fused != 0);
+        if (rc) return rc;
+    }
     rc = fo_gemm_signal(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, MM, RA, monitor, algo,
                         h->gemm_stream);
     if (rc) return rc;  // nothing has been enqueued on the consumer stream yet
@@ -263,11 +280,11 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
             long tiles = 0;
             for (int g = i; g < j; g++) tiles += cseg_host[g];
             const int64_t n = tiles * tile_elems;
-            rc = j - i == 1 ? fo_wait(cseg_host[i], MM + i, h->comm_stream)  // resets the counter
-                            : fo_wait_groups(j - i, cseg_dev + i, MM + i, h->comm_stream);
+            rc = j - i == 1 ? fo_wait(cseg_host[i], MM + i, cstream)  // resets the counter
+                            : fo_wait_groups(j - i, cseg_dev + i, MM + i, cstream);
             if (rc) return rc;
             if (acc) {  // the groups of a batch are one contiguous range
-                rc = fo_consumer_reduce(dtype, c + off, acc + off, n, h->comm_stream);
+                rc = fo_consumer_reduce(dtype, c + off, acc + off, n, cstream);
                 if (rc) return rc;
             }
             off += n;
@@ -275,7 +292,7 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
             i = j;
         }
     }
-    return join(h, captured);
+    return same_stream ? FO_OK : join(h, captured);
 }
 
 extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, int N, int K,
@@ -298,15 +315,21 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
     const int64_t seg_stride = (int64_t)M * N / W;
     if (h->acc && h->acc_nelem < (int64_t)M * N) return FO_ERR_ARG;
 
-    const int fused = fused_grid(h, G);
+    const bool same_stream = in_stream(h, M, N, K);
+    const int fused = same_stream ? 0 : fused_grid(h, G);
+    fo_stream_t cstream = same_stream ? h->gemm_stream : h->comm_stream;
     int32_t wave = 0;
-    if (!fused) {
+    if (same_stream) {
+        wave = TM * TN;  // every group in one batch
+    } else if (!fused) {
         rc = fo_gemm_wave_tiles(dtype, algo, M, N, &wave);
         if (rc) return rc;
     }
     const bool captured = capturing(h);
-    rc = fork(h, captured, fused != 0);
-    if (rc) return rc;
+    if (!same_stream) {
+        rc = fork(h, captured, fused != 0);
+        if (rc) return rc;
+    }
     rc = fo_gemm_scatter(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, MM, RA, RE, monitor, algo,
                          h->gemm_stream);
     if (rc) return rc;
@@ -322,7 +345,7 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
         rc = fo_wait_reduce_groups(dtype, C, h->acc, MM, cseg_dev, G, tile_elems, W, seg_stride,
                                    own_in_consumer ? D : nullptr, h->rank, h->workspace, fused,
                                    fused_slices((int64_t)M * N, G, fused), fused_poll_gap_ns(M, N, K, fused),
-                                   h->comm_stream);
+                                   cstream);
         if (rc) return rc;
     }
     int64_t off = 0;
@@ -330,8 +353,8 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
     for (int i = 0; i < G;) {
         const int j = fused ? i + 1 : batch_end(cseg_host, G, i, done, wave);
         if (!fused) {
-            rc = j - i == 1 ? fo_wait(cseg_host[i], MM + i, h->comm_stream)
-                            : fo_wait_groups(j - i, cseg_dev + i, MM + i, h->comm_stream);
+            rc = j - i == 1 ? fo_wait(cseg_host[i], MM + i, cstream)
+                            : fo_wait_groups(j - i, cseg_dev + i, MM + i, cstream);
             if (rc) return rc;
         }
         if (!fused && acc && W > 1 && j - i > 1) {
@@ -340,26 +363,26 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
             for (int g = i; g < j; g++) most = cseg_host[g] > most ? cseg_host[g] : most;
             rc = fo_consumer_reduce_rs_groups(dtype, c + off, acc + off / W, cseg_dev + i, j - i, most, tile_elems,
                                               W, seg_stride, own_in_consumer ? d + off / W : nullptr, h->rank,
-                                              h->comm_stream);
+                                              cstream);
             if (rc) return rc;
         }
         for (int g = i; g < j; g++) {
             const int64_t n = cseg_host[g] * tile_elems;
             if (!fused && acc && !(W > 1 && j - i > 1)) {
                 rc = fo_consumer_reduce_rs_own(dtype, c + off, acc + off / W, n, W, seg_stride,
-                                               own_in_consumer ? d + off / W : nullptr, h->rank, h->comm_stream);
+                                               own_in_consumer ? d + off / W : nullptr, h->rank, cstream);
                 if (rc) return rc;
             }
             if (d && !own_in_consumer)
                 FO_HIP_CHECK(hipMemcpyAsync(d + off / W, c + off + (int64_t)h->rank * (n / W),
                                             (size_t)(n / W) * 2, hipMemcpyDeviceToDevice,
-                                            h->comm_stream));
+                                            static_cast<hipStream_t>(cstream)));
             off += n;
             done += cseg_host[g];
         }
         i = j;
     }
-    return join(h, captured);
+    return same_stream ? FO_OK : join(h, captured);
 }
 
 extern "C" int fo_overlap_gemm_allreduce_serial(fo_overlap_t *h, int dtype, int M, int N, int K,

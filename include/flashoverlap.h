@@ -213,8 +213,12 @@ int fo_overlap_set_accumulator(fo_overlap_t *h, void *acc, int64_t nelem);
  * at the end (room for G + 1 entries); returns n, or a negative error.
  * wave_tiles <= 0: no batching. */
 int fo_overlap_plan_batches(const int32_t *cseg_host, int G, int wave_tiles, int32_t *first);
-/* fused < 0 (default): chosen per call, one launch when there are more than 16
- * groups; 0: always 2*G launches as the reference's host loop
+/* fused < 0 (default): chosen per call.  A GEMM below 6.4e10 flop (about 50 us)
+ * keeps the whole call on the GEMM stream (signal GEMM, one wait over all
+ * groups, one consumer launch: nothing that short can hide a fork and a join);
+ * otherwise one launch when there are more than 16 groups, else per-wave
+ * launches.  0: always the second stream with wait + consumer launches per
+ * group (per GEMM wave) as the reference's host loop
  * (src/overlap_impl.cu:250-258); 1: always one fo_wait_reduce_groups launch
  * with the default grid; n > 1: the same with n workgroups. */
 int fo_overlap_set_fused_consumer(fo_overlap_t *h, int fused);

@@ -27,7 +27,7 @@ def _setup(fo, dtype, bm, bn, M, N, K, cseg, swizzle=1, seed=50, hint=None):
     return algo, RA, A, B, Ab, Bb, MM, cseg_cpu, cseg_cpu.cuda()
 
 
-@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("fused", [False, True, -1])   # -1: automatic; this short GEMM then stays on one stream
 @pytest.mark.parametrize("dtype", [F16, BF16])
 def test_allreduce_overlap_against_checker(fo, oracle, dtype, fused):
     bm, bn, M, N, K = 128, 128, 1024, 1024, 256
@@ -69,7 +69,7 @@ def test_allreduce_overlap_against_checker(fo, oracle, dtype, fused):
     ov.close()
 
 
-@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("fused", [False, True, -1])
 def test_reducescatter_overlap_segments(fo, oracle, fused):
     dtype, W, rank = F16, 4, 2
     bm, bn, M, N, K = 128, 128, 1024, 512, 128
