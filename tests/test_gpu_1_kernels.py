@@ -333,7 +333,7 @@ def test_error_codes_on_gpu(fo):
 
 
 def test_reorder_table_changed_in_place_between_launches(fo):
-    """RA and cSeg are read through the scalar cache / an LDS table built at kernel start:
+    """RA is read through the scalar cache, cSeg into registers at kernel start:
     a launch must see what the tensors hold at that time, not what an earlier launch read."""
     bm, bn, M, N, K = 128, 128, 2048, 2048, 128
     algo = _algo(fo, bm, bn, swizzle=4)
