@@ -88,6 +88,10 @@ struct fo_raster {
     int grid_m, grid_n;  // macro tiles along M and N
     int panel;           // raster panel height in macro tiles
     int xcd_remap;       // 1: workgroup id is de-interleaved over the 8 XCDs
+    // A last wave of 256x256 tiles that would leave most CUs idle is computed by a
+    // second launch instead, with the Algo's own (smaller) tile: the last
+    // tail_tiles positions of the raster, each cut into tail_sub_m x tail_sub_n.
+    int tail_tiles, tail_sub_m, tail_sub_n;
 };
 int fo_pick_raster(int algo, int M, int N, fo_raster *r);
 
@@ -111,4 +115,20 @@ __host__ __device__ inline void fo_wg_to_tile(int wg, int grid_m, int grid_n, in
     int in = v - p * per_panel;
     *pm = first_m + in % rows;
     *pn = in / rows;
+}
+
+// Unit u of a launch that covers raster positions first, first + 1, ... with each
+// position cut into sub_m x sub_n tiles of its own -> coordinates in those tiles.
+__host__ __device__ inline void fo_unit_to_tile(int u, int first, int sub_m, int sub_n, int grid_m,
+                                                int grid_n, int panel, int xcd_remap, int *pm, int *pn) {
+    const int per = sub_m * sub_n;
+    if (per == 1) {
+        fo_wg_to_tile(first + u, grid_m, grid_n, panel, xcd_remap, pm, pn);
+        return;
+    }
+    int ppm, ppn;
+    fo_wg_to_tile(first + u / per, grid_m, grid_n, panel, xcd_remap, &ppm, &ppn);
+    const int s = u % per;
+    *pm = ppm * sub_m + s / sub_n;
+    *pn = ppn * sub_n + s % sub_n;
 }

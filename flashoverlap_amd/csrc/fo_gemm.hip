@@ -31,7 +31,7 @@ int launch_variant(const GemmArgs &a, hipStream_t stream, int *resident_out) {
         resident = (cus * per_cu) / 8 * 8;
         if (resident <= 0) resident = cus * per_cu;
     }
-    const int ntiles = a.grid_m * a.grid_n;
+    const int ntiles = a.count;
     if (resident_out) {
         *resident_out = ntiles < resident ? ntiles : resident;
         return FO_OK;
@@ -89,6 +89,8 @@ int run_gemm(int mode, int dtype, int M, int N, int K, int rLDN, const int32_t *
     a.rLDN = rLDN;
     a.RA = RA; a.RE = RE; a.cseg = cseg; a.G = G; a.MM = MM; a.monitor = monitor;
     a.grid_m = r.grid_m; a.grid_n = r.grid_n; a.panel = r.panel; a.xcd_remap = r.xcd_remap;
+    a.first = 0; a.sub_m = a.sub_n = 1;
+    a.count = r.grid_m * r.grid_n - r.tail_tiles;
     if (mode != MODE_PLAIN) {
         const long T = (long)(M / a.BM) * a.TN;
         if (!MM || !RA || !cseg) return FO_ERR_ARG;
@@ -98,11 +100,21 @@ int run_gemm(int mode, int dtype, int M, int N, int K, int rLDN, const int32_t *
         if (monitor && G > a.TN - 1) return FO_ERR_SEGMENTS;
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    switch (mode) {
-        case MODE_PLAIN: return launch_dtype<MODE_PLAIN>(dtype, a, r.mtm, r.mtn, s);
-        case MODE_SIGNAL: return launch_dtype<MODE_SIGNAL>(dtype, a, r.mtm, r.mtn, s);
-        default: return launch_dtype<MODE_SCATTER>(dtype, a, r.mtm, r.mtn, s);
-    }
+    auto launch = [&](const GemmArgs &g, int mtm, int mtn) {
+        switch (mode) {
+            case MODE_PLAIN: return launch_dtype<MODE_PLAIN>(dtype, g, mtm, mtn, s);
+            case MODE_SIGNAL: return launch_dtype<MODE_SIGNAL>(dtype, g, mtm, mtn, s);
+            default: return launch_dtype<MODE_SCATTER>(dtype, g, mtm, mtn, s);
+        }
+    };
+    rc = launch(a, r.mtm, r.mtn);
+    if (rc || !r.tail_tiles) return rc;
+    // the last, partial wave of 256x256 tiles: the same raster positions in the Algo's own tile
+    GemmArgs t = a;
+    t.first = a.count;
+    t.sub_m = r.tail_sub_m; t.sub_n = r.tail_sub_n;
+    t.count = r.tail_tiles * r.tail_sub_m * r.tail_sub_n;
+    return launch(t, a.BM, a.BN);
 }
 
 }  // namespace
@@ -117,6 +129,7 @@ extern "C" int fo_gemm_wave_tiles(int dtype, int algo, int M, int N, int32_t *ti
     GemmArgs a = {};
     a.grid_m = r.grid_m;
     a.grid_n = r.grid_n;
+    a.count = r.grid_m * r.grid_n - r.tail_tiles;
     int resident = 0;
     rc = launch_dtype<MODE_SIGNAL>(dtype, a, r.mtm, r.mtn, nullptr, &resident);
     if (rc) return rc;

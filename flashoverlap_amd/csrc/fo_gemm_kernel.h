@@ -58,7 +58,8 @@ struct GemmArgs {
     int G;
     int32_t *MM;
     int monitor;
-    int grid_m, grid_n, panel, xcd_remap;
+    int grid_m, grid_n, panel, xcd_remap;  // the raster of this launch's parent tiles
+    int first, sub_m, sub_n, count;        // this launch: positions from `first`, each cut into sub_m x sub_n macro tiles, `count` of them
 };
 
 constexpr int kMaxSub = 4;        // reorder tiles per macro tile (256x256 over 128x128)
@@ -175,7 +176,7 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
-    const int ntiles = p.grid_m * p.grid_n;
+    const int ntiles = p.count;
     // K is a multiple of 8 (one 16-byte chunk).  A last K step that is not full
     // is loaded with its out-of-range chunks redirected to the step's first
     // chunk (valid memory) and zeroed in LDS before the stage is published.
@@ -482,7 +483,7 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
     // ---- persistent loop over this workgroup's macro tiles
     int tile = blockIdx.x;
     int pm, pn;
-    fo_wg_to_tile(tile, p.grid_m, p.grid_n, p.panel, p.xcd_remap, &pm, &pn);
+    fo_unit_to_tile(tile, p.first, p.sub_m, p.sub_n, p.grid_m, p.grid_n, p.panel, p.xcd_remap, &pm, &pn);
     pm = __builtin_amdgcn_readfirstlane(pm);
     pn = __builtin_amdgcn_readfirstlane(pn);
     set_tile(pm, pn);
@@ -588,7 +589,7 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
         const int next = tile + gridDim.x;
         const bool has_next = next < ntiles;
         if (has_next) {
-            fo_wg_to_tile(next, p.grid_m, p.grid_n, p.panel, p.xcd_remap, &pm, &pn);
+            fo_unit_to_tile(next, p.first, p.sub_m, p.sub_n, p.grid_m, p.grid_n, p.panel, p.xcd_remap, &pm, &pn);
             pm = __builtin_amdgcn_readfirstlane(pm);
             pn = __builtin_amdgcn_readfirstlane(pn);
             set_tile(pm, pn);

@@ -61,6 +61,27 @@ def test_algo_table_matches_reference_rows():
     assert _capi.find_algo(128, 256, swizzle=4) == 57
 
 
+def test_schedule_order_with_a_partial_last_wave():
+    """1089 workgroup tiles of 256x256 on 256 workgroups leave 65 for a fifth wave; those are walked
+    in the Algo's own tile by a second launch, and the analytic hint must follow: a permutation of all
+    reorder tiles whose last 65 * 4 entries are exactly the 128x128 tiles of the last 65 positions."""
+    algo = _capi.find_algo(128, 128, swizzle=4)
+    M = N = 8448
+    order = _capi.schedule_order(algo, M, N)
+    T = (M // 128) * (N // 128)
+    assert sorted(order) == list(range(T))
+    whole = _capi.schedule_order(_capi.find_algo(128, 128, swizzle=4), 8192, 8192)   # 1024 tiles: no tail
+    assert sorted(whole) == list(range(64 * 64))
+    # every group of four consecutive entries in the main part is one 256x256 tile
+    tn = N // 128
+    for i in range(0, (1089 - 65) * 4, 4):
+        a, b, c, d = order[i:i + 4]
+        assert b == a + 1 and c == a + tn and d == c + 1 and (a // tn) % 2 == 0 and (a % tn) % 2 == 0
+    # 256x128 reorder tiles: two per position, tail cut in two
+    order2 = _capi.schedule_order(_capi.find_algo(256, 128, swizzle=4), M, N)
+    assert sorted(order2) == list(range((M // 256) * (N // 128)))
+
+
 def test_argument_validation_without_gpu():
     L = _capi.lib()
     null = ctypes.c_void_p()
