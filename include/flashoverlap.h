@@ -52,13 +52,16 @@ int fo_algo_info(int algo, int32_t info[12]);
 /* Tile issue order of the GEMM kernels: order[s] = id (tm*TN + tn) of the
  * s-th BM x BN tile in workgroup dispatch order.  It is the analytic
  * counterpart of the hint that tune/search.py:83-157 measures in monitor
- * mode; order must hold (M/BM)*(N/BN) ints (host memory). */
+ * mode; order must hold (M/BM)*(N/BN) ints (host memory).  Where the last
+ * wave of 256x256 workgroup tiles is at most half full, those tiles are
+ * computed by a second launch in BM x BN tiles; the order lists them last. */
 int fo_schedule_order(int algo, int M, int N, int32_t *order);
 
 /* How the GEMM kernels cover the problem: reorder tiles per workgroup (the
  * workgroup tile may span several BM x BN tiles) and the number of workgroups.
  * One wave of the 256-CU chip completes 256 * tiles_per_workgroup tiles; the
- * reference's tuner uses sm_count - 2 tiles per wave (tune/search.py:404). */
+ * reference's tuner uses sm_count - 2 tiles per wave (tune/search.py:404).
+ * Both numbers describe the main launch's tiling of the whole problem. */
 int fo_workgroup_tiles(int algo, int M, int N, int32_t *tiles_per_workgroup, int32_t *workgroups);
 /* Reorder tiles that complete together: the workgroups the persistent GEMM
  * keeps resident on the current device times the reorder tiles per workgroup
