@@ -584,18 +584,23 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
 
-        // request the next tile's first stage; it lands during the epilogue
+        // The next tile's first stage is requested before the epilogue and lands
+        // while it runs.  (Scatter epilogue: after its row map entries have
+        // arrived, so that their wait does not include these loads.)
         const int cur_pm = pm, cur_pn = pn;
         const int next = tile + gridDim.x;
         const bool has_next = next < ntiles;
-        if (has_next) {
-            fo_unit_to_tile(next, p.first, p.sub_m, p.sub_n, p.grid_m, p.grid_n, p.panel, p.xcd_remap, &pm, &pn);
-            pm = __builtin_amdgcn_readfirstlane(pm);
-            pn = __builtin_amdgcn_readfirstlane(pn);
-            set_tile(pm, pn);
-            issue_a_any(0, 0);
-            issue_b_any(0, 0);
-        }
+        auto request_next = [&]() {
+            if (has_next) {
+                fo_unit_to_tile(next, p.first, p.sub_m, p.sub_n, p.grid_m, p.grid_n, p.panel, p.xcd_remap, &pm, &pn);
+                pm = __builtin_amdgcn_readfirstlane(pm);
+                pn = __builtin_amdgcn_readfirstlane(pn);
+                set_tile(pm, pn);
+                issue_a_any(0, 0);
+                issue_b_any(0, 0);
+            }
+        };
+        if (MODE != MODE_SCATTER) request_next();
 
         // ---- epilogue: accumulators -> 16-bit -> LDS (per-wave strip of 32 rows) -> global
         // A wavefront's WTM x WTN block lies inside one reorder tile (BM and BN
@@ -630,6 +635,8 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
 #pragma unroll
                     for (int ps = 0; ps < 32 / RPP; ps++)
                         dest_row[i * (32 / RPP) + ps] = p.RE[trow + i * 32 + ps * RPP + srow];
+                wait_vmcnt<0>();
+                request_next();
             }
 #pragma unroll
             for (int i = 0; i < FMB; i++) {  // 32 output rows = two rows of accumulator blocks
