@@ -22,6 +22,7 @@ SIGNATURES = {
     "fo_schedule_order": (c_int, [c_int, c_int, c_int, vp]),
     "fo_workgroup_tiles": (c_int, [c_int, c_int, c_int, vp, vp]),
     "fo_gemm_wave_tiles": (c_int, [c_int, c_int, c_int, c_int, vp]),
+    "fo_gemm_kernel_info": (c_int, [c_int, c_int, c_int, c_int, c_int, vp]),
     "fo_set": (c_int, [vp, c_int, vp]),
     "fo_wait_groups": (c_int, [c_int, vp, vp, vp]),
     "fo_gemm": (c_int, [c_int, c_int, c_int, c_int, vp, vp, vp, c_int, vp]),
@@ -131,6 +132,14 @@ def wave_tiles(algo, M, N, dtype=F16):
     tiles = ctypes.c_int32()
     check(lib().fo_gemm_wave_tiles(int(dtype), int(algo), M, N, ctypes.byref(tiles)), "fo_gemm_wave_tiles")
     return tiles.value
+
+
+def kernel_info(algo, M, N, epilogue=1, dtype=F16):
+    """{resident workgroups, vector registers per lane, LDS bytes, threads} of the main GEMM launch
+    for this problem (epilogue 0 plain, 1 signal, 2 scatter); asks the GPU."""
+    info = (ctypes.c_int32 * 4)()
+    check(lib().fo_gemm_kernel_info(int(dtype), int(algo), M, N, int(epilogue), info), "fo_gemm_kernel_info")
+    return {"resident": info[0], "vgprs": info[1], "lds_bytes": info[2], "threads": info[3]}
 
 
 def plan_batches(cseg, wave_tiles):

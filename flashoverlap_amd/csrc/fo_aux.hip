@@ -79,8 +79,8 @@ constexpr int CONSUMER_THREADS = 256;
 constexpr int CONSUMER_UNROLL = 4;
 constexpr int CONSUMER_MAX_BLOCKS = 256;  // a spinning grid of this size cannot occupy every CU three-deep
 // __launch_bounds__(256, 8) below caps the kernels at 64 VGPRs: the signalling GEMM holds two
-// wavefronts of up to 224 registers on each SIMD (208 as built), which leaves at least 64 of the 512
-// for one consumer wavefront.
+// wavefronts of up to 224 registers on each SIMD, which leaves 64 of the 512 for one consumer
+// wavefront.
 
 // 16-byte load that bypasses the non-coherent caches (system-scope cache
 // policy).  The fused consumer reads tiles that workgroups on other XCDs wrote

@@ -11,7 +11,8 @@ using namespace fo_gemm_dev;
 // workgroups as the device keeps resident at once (or fewer, if the problem has
 // fewer macro tiles); each walks the raster with that stride.
 // With `resident_out` set nothing is launched: the call only reports how many workgroups the
-// launch would hold.
+// launch would hold, and in resident_out[1..3] the kernel's registers per lane, LDS bytes
+// and threads per workgroup.
 template <typename Tag, int MTM, int MTN, int BK, int SA, int SB, int WM, int WN, int MODE>
 int launch_variant(const GemmArgs &a, hipStream_t stream, int *resident_out) {
     auto kern = fo_gemm_kernel<Tag, MTM, MTN, BK, SA, SB, WM, WN, MODE>;
@@ -33,7 +34,12 @@ int launch_variant(const GemmArgs &a, hipStream_t stream, int *resident_out) {
     }
     const int ntiles = a.count;
     if (resident_out) {
-        *resident_out = ntiles < resident ? ntiles : resident;
+        hipFuncAttributes attr;
+        FO_HIP_CHECK(hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(kern)));
+        resident_out[0] = ntiles < resident ? ntiles : resident;
+        resident_out[1] = attr.numRegs;
+        resident_out[2] = smem;
+        resident_out[3] = threads;
         return FO_OK;
     }
     dim3 grid(ntiles < resident ? ntiles : resident), block(threads);
@@ -130,10 +136,31 @@ extern "C" int fo_gemm_wave_tiles(int dtype, int algo, int M, int N, int32_t *ti
     a.grid_m = r.grid_m;
     a.grid_n = r.grid_n;
     a.count = r.grid_m * r.grid_n - r.tail_tiles;
-    int resident = 0;
-    rc = launch_dtype<MODE_SIGNAL>(dtype, a, r.mtm, r.mtn, nullptr, &resident);
+    int info[4] = {0, 0, 0, 0};
+    rc = launch_dtype<MODE_SIGNAL>(dtype, a, r.mtm, r.mtn, nullptr, info);
     if (rc) return rc;
-    *tiles = resident * (r.mtm / e->f[0]) * (r.mtn / e->f[1]);
+    *tiles = info[0] * (r.mtm / e->f[0]) * (r.mtn / e->f[1]);
+    return FO_OK;
+}
+
+extern "C" int fo_gemm_kernel_info(int dtype, int algo, int M, int N, int epilogue, int32_t info[4]) {
+    if (!info) return FO_ERR_ARG;
+    fo_raster r;
+    int rc = fo_pick_raster(algo, M, N, &r);
+    if (rc) return rc;
+    GemmArgs a = {};
+    a.grid_m = r.grid_m;
+    a.grid_n = r.grid_n;
+    a.count = r.grid_m * r.grid_n - r.tail_tiles;
+    int out[4] = {0, 0, 0, 0};
+    switch (epilogue) {
+        case MODE_PLAIN: rc = launch_dtype<MODE_PLAIN>(dtype, a, r.mtm, r.mtn, nullptr, out); break;
+        case MODE_SIGNAL: rc = launch_dtype<MODE_SIGNAL>(dtype, a, r.mtm, r.mtn, nullptr, out); break;
+        case MODE_SCATTER: rc = launch_dtype<MODE_SCATTER>(dtype, a, r.mtm, r.mtn, nullptr, out); break;
+        default: return FO_ERR_ARG;
+    }
+    if (rc) return rc;
+    for (int i = 0; i < 4; i++) info[i] = out[i];
     return FO_OK;
 }
 

@@ -386,10 +386,11 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
     // fetched right behind row r into the registers row r - 1 used.  The B
     // fragments of an MFMA k-step are live for its FM rows; the next k-step's are
     // fetched during its last FN rows into a second set.
-    constexpr int AHEAD = 3, ARING = AHEAD + 1;
+    constexpr int AHEAD = (FM >= 8 ? 7 : 3), ARING = AHEAD + 1;
     // The step's P direct-to-LDS loads are dealt over the rows behind its barrier
-    // instead of being issued in one burst (measured: 3 % faster; AHEAD = 7 with
-    // the loads over eight rows another 0.7 %, for 16 more registers).
+    // instead of being issued in one burst (measured: 3 % faster over four rows
+    // with AHEAD = 3; AHEAD = 7 with the loads over eight rows another 0.7-1 %,
+    // for 16 more registers, where a k-step has eight A fragments).
     constexpr int DMA_ROWS = AHEAD + 1;
     constexpr int ROWS = KK * FM;
     static_assert(FM % ARING == 0 && FN <= FM && AHEAD < FM, "row pipeline");

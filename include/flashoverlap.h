@@ -68,6 +68,13 @@ int fo_workgroup_tiles(int algo, int M, int N, int32_t *tiles_per_workgroup, int
  * (needs a GPU: the count comes from the occupancy of the compiled kernel).
  * The counterpart of sm_count - 2 in tune/search.py:404. */
 int fo_gemm_wave_tiles(int dtype, int algo, int M, int N, int32_t *tiles);
+/* What the main launch of a problem occupies on the device (needs a GPU; no
+ * counterpart in the reference): info = {resident workgroups, vector
+ * registers per lane, LDS bytes per workgroup, threads per workgroup} of the
+ * kernel with the given epilogue (0 plain, 1 signal, 2 scatter).  The consumer
+ * kernels are built for one 64-register wavefront per SIMD beside two GEMM
+ * wavefronts: that holds while the register count stays at or below 224. */
+int fo_gemm_kernel_info(int dtype, int algo, int M, int N, int epilogue, int32_t info[4]);
 
 /* ---- GEMM -------------------------------------------------------------
  * C[M,N] = A[M,K] . B[N,K]^T, 16-bit in/out, fp32 accumulate.

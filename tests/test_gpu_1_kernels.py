@@ -318,6 +318,18 @@ def test_reorder_rmsnorm_undoes_the_permutation(fo, oracle, dtype):
         assert max_rel_err(Y.cpu(), rmsnorm_f64(plain, Wt, 1e-6)) <= REL_TOL
 
 
+@pytest.mark.parametrize("dtype", [F16, BF16])
+def test_gemm_leaves_registers_for_a_consumer_wavefront(fo, dtype):
+    """The consumer kernels are built for one 64-register wavefront per SIMD beside the two
+    wavefronts of a signalling GEMM workgroup: 2 x GEMM registers (allocated in eights) + 64 must
+    fit the 512 of a SIMD, or the overlapped path silently degrades into a serial one."""
+    algo = _algo(fo, 128, 256, swizzle=4)
+    for epilogue in (1, 2):
+        info = fo._capi.kernel_info(algo, 8192, 8192, epilogue=epilogue, dtype=dtype)
+        assert info["resident"] == 256 and info["threads"] == 512 and info["lds_bytes"] <= 160 * 1024
+        assert 2 * ((info["vgprs"] + 7) // 8 * 8) + 64 <= 512, info
+
+
 def test_error_codes_on_gpu(fo):
     A = torch.zeros(128, 64, device="cuda", dtype=torch.float16)
     C = torch.zeros(128, 128, device="cuda", dtype=torch.float16)
