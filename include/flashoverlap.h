@@ -120,9 +120,10 @@ int fo_wait(int expect, int32_t *counter, fo_stream_t stream);
  * success *status is left unchanged.  No counterpart in the reference (its
  * waiter spins forever); exists so that failure handling can be tested
  * without hanging a GPU. */
-/* fo_wait for `count` consecutive groups in one launch: for g = 0..count-1 in
- * turn, spin until counters[g] == expect_dev[g] (device array, e.g. cSEG_GPU + i),
- * then reset counters[g].  Used for groups that complete in the same wave of the
+/* fo_wait for `count` consecutive groups in one launch: for every g in
+ * 0..count-1 (a lane per group, side by side), spin until counters[g] ==
+ * expect_dev[g] (device array, e.g. cSEG_GPU + i), then reset counters[g]; the
+ * kernel ends when all have been reset.  Used for groups that complete in the same wave of the
  * GEMM, where one launch per group would only add launch latency. */
 int fo_wait_groups(int count, const int32_t *expect_dev, int32_t *counters, fo_stream_t stream);
 /* One-lane kernel that stores value into *word.  With fo_wait(value, word, other_stream)
