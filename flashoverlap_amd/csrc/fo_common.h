@@ -95,6 +95,12 @@ struct fo_raster {
 };
 int fo_pick_raster(int algo, int M, int N, fo_raster *r);
 
+// fo_gemm_signal / fo_gemm_scatter (RE != nullptr) without the counters: tiles are
+// stored reordered, MM is never touched (fo_gemm.hip; used by fo_overlap.cpp).
+int fo_gemm_reordered_quiet(int dtype, int M, int N, int K, int rLDN, const int32_t *cseg_dev, int G,
+                            const void *A, const void *B, void *C, const int32_t *RA, const int32_t *RE,
+                            int algo, fo_stream_t stream);
+
 // Workgroup id -> macro tile coordinates; identical code on host and device.
 __host__ __device__ inline void fo_wg_to_tile(int wg, int grid_m, int grid_n, int panel,
                                               int xcd_remap, int *pm, int *pn) {

@@ -73,7 +73,7 @@ int launch_dtype(int dtype, const GemmArgs &a, int mtm, int mtn, hipStream_t str
 
 int run_gemm(int mode, int dtype, int M, int N, int K, int rLDN, const int32_t *cseg, int G,
              const void *A, const void *B, void *C, int32_t *MM, const int32_t *RA,
-             const int32_t *RE, int monitor, int algo, fo_stream_t stream) {
+             const int32_t *RE, int monitor, int algo, fo_stream_t stream, bool quiet = false) {
     if (dtype != FO_F16 && dtype != FO_BF16) return FO_ERR_DTYPE;
     const fo_algo_entry *e = fo_algo_lookup(algo);
     if (!e) return FO_ERR_ALGO;
@@ -97,9 +97,10 @@ int run_gemm(int mode, int dtype, int M, int N, int K, int rLDN, const int32_t *
     a.grid_m = r.grid_m; a.grid_n = r.grid_n; a.panel = r.panel; a.xcd_remap = r.xcd_remap;
     a.first = 0; a.sub_m = a.sub_n = 1;
     a.count = r.grid_m * r.grid_n - r.tail_tiles;
+    a.quiet = quiet ? 1 : 0;
     if (mode != MODE_PLAIN) {
         const long T = (long)(M / a.BM) * a.TN;
-        if (!MM || !RA || !cseg) return FO_ERR_ARG;
+        if ((!MM && !quiet) || !RA || !cseg) return FO_ERR_ARG;
         if (mode == MODE_SCATTER && !RE) return FO_ERR_ARG;
         if (rLDN <= 0 || T % rLDN) return FO_ERR_SHAPE;
         if (G <= 0 || G > T) return FO_ERR_SEGMENTS;
@@ -124,6 +125,15 @@ int run_gemm(int mode, int dtype, int M, int N, int K, int rLDN, const int32_t *
 }
 
 }  // namespace
+
+// The reordered (optionally row-mapped) store of the signalling GEMMs without
+// their counters, for a caller that orders GEMM and consumer by the stream alone.
+int fo_gemm_reordered_quiet(int dtype, int M, int N, int K, int rLDN, const int32_t *cseg_dev, int G,
+                            const void *A, const void *B, void *C, const int32_t *RA, const int32_t *RE,
+                            int algo, fo_stream_t stream) {
+    return run_gemm(RE ? MODE_SCATTER : MODE_SIGNAL, dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, nullptr, RA, RE,
+                    0, algo, stream, true);
+}
 
 extern "C" int fo_gemm_wave_tiles(int dtype, int algo, int M, int N, int32_t *tiles) {
     if (!tiles) return FO_ERR_ARG;

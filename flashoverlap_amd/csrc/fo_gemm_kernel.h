@@ -60,6 +60,7 @@ struct GemmArgs {
     int monitor;
     int grid_m, grid_n, panel, xcd_remap;  // the raster of this launch's parent tiles
     int first, sub_m, sub_n, count;        // this launch: positions from `first`, each cut into sub_m x sub_n macro tiles, `count` of them
+    int quiet;                             // signalling epilogues: store the tiles reordered, touch no counter
 };
 
 constexpr int kMaxSub = 4;        // reorder tiles per macro tile (256x256 over 128x128)
@@ -323,7 +324,8 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
 #pragma unroll
     for (int q = 0; q < NPRE; q++) pre[q] = 0;
     const bool reg_search = p.G <= kPrefixRegs;
-    if (MODE != MODE_PLAIN && reg_search) {
+    const bool signalling = MODE != MODE_PLAIN && !p.quiet;
+    if (signalling && reg_search) {
         int base = 0;
 #pragma unroll
         for (int q = 0; q < NPRE; q++) {
@@ -462,7 +464,7 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
                     __builtin_amdgcn_s_barrier();
                     asm volatile("" ::: "memory");
                     if (!STEADY && MODE != MODE_PLAIN) {
-                        if (first && owed && wave == 0) announce(prev_rs, prev_gs);
+                        if (first && owed && wave == 0) announce(prev_rs, prev_gs);  // never owed when quiet
                     }
                     if constexpr (!STEADY) {
                         if (kt + SB < KT) issue_b_any(kt + SB, sb);
@@ -681,7 +683,7 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
             }
         }
 
-        if (MODE != MODE_PLAIN) {
+        if (signalling) {
             int gs[kMaxSub] = {0, 0, 0, 0};
             if (wave == 0) groups_of(rs, gs);
             if (has_next && KT >= 2) {

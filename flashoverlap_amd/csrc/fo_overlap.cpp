@@ -27,8 +27,9 @@ namespace {
 constexpr int kFusedFromGroups = 16;
 
 // In automatic mode a GEMM shorter than this many flop (about 50 us of this
-// GPU) keeps the whole call on the GEMM stream: signal GEMM, one wait that
-// resets every counter, one consumer launch.  Fork, join and pollers beside the
+// GPU) keeps the whole call on the GEMM stream: the GEMM with its reordered
+// store and one consumer launch (with the monitor on: the signalling GEMM and
+// one wait that resets every counter between them).  Fork, join and pollers beside the
 // GEMM cost more than such a GEMM can hide (4096x4096x512 with 256 groups:
 // 71 us overlapped, 48 us in stream).
 constexpr double kInStreamBelowFlop = 6.4e10;
@@ -261,8 +262,15 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
         rc = fork(h, captured, fused != 0);
         if (rc) return rc;
     }
-    rc = fo_gemm_signal(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, MM, RA, monitor, algo,
-                        h->gemm_stream);
+    // On one stream the order of the launches is all the synchronisation there is
+    // to do: unless the caller wants the monitor's stamps, the GEMM then leaves
+    // the counters alone (they stay zero, as the waits would have left them).
+    const bool quiet = same_stream && !monitor;
+    if (!MM) return FO_ERR_ARG;
+    rc = quiet ? fo_gemm_reordered_quiet(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, RA, nullptr, algo,
+                                         h->gemm_stream)
+               : fo_gemm_signal(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, MM, RA, monitor, algo,
+                                h->gemm_stream);
     if (rc) return rc;  // nothing has been enqueued on the consumer stream yet
 
     if (fused) {
@@ -280,9 +288,11 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
             long tiles = 0;
             for (int g = i; g < j; g++) tiles += cseg_host[g];
             const int64_t n = tiles * tile_elems;
-            rc = j - i == 1 ? fo_wait(cseg_host[i], MM + i, cstream)  // resets the counter
-                            : fo_wait_groups(j - i, cseg_dev + i, MM + i, cstream);
-            if (rc) return rc;
+            if (!quiet) {
+                rc = j - i == 1 ? fo_wait(cseg_host[i], MM + i, cstream)  // resets the counter
+                                : fo_wait_groups(j - i, cseg_dev + i, MM + i, cstream);
+                if (rc) return rc;
+            }
             if (acc) {  // the groups of a batch are one contiguous range
                 rc = fo_consumer_reduce(dtype, c + off, acc + off, n, cstream);
                 if (rc) return rc;
@@ -330,8 +340,12 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
         rc = fork(h, captured, fused != 0);
         if (rc) return rc;
     }
-    rc = fo_gemm_scatter(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, MM, RA, RE, monitor, algo,
-                         h->gemm_stream);
+    const bool quiet = same_stream && !monitor;  // as in fo_overlap_gemm_allreduce
+    if (!MM || !RE) return FO_ERR_ARG;
+    rc = quiet ? fo_gemm_reordered_quiet(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, RA, RE, algo,
+                                         h->gemm_stream)
+               : fo_gemm_scatter(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, MM, RA, RE, monitor, algo,
+                                 h->gemm_stream);
     if (rc) return rc;
 
     uint16_t *c = static_cast<uint16_t *>(C);
@@ -352,7 +366,7 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
     long done = 0;
     for (int i = 0; i < G;) {
         const int j = fused ? i + 1 : batch_end(cseg_host, G, i, done, wave);
-        if (!fused) {
+        if (!fused && !quiet) {
             rc = j - i == 1 ? fo_wait(cseg_host[i], MM + i, cstream)
                             : fo_wait_groups(j - i, cseg_dev + i, MM + i, cstream);
             if (rc) return rc;

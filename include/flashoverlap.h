@@ -225,8 +225,10 @@ int fo_overlap_set_accumulator(fo_overlap_t *h, void *acc, int64_t nelem);
  * wave_tiles <= 0: no batching. */
 int fo_overlap_plan_batches(const int32_t *cseg_host, int G, int wave_tiles, int32_t *first);
 /* fused < 0 (default): chosen per call.  A GEMM below 6.4e10 flop (about 50 us)
- * keeps the whole call on the GEMM stream (signal GEMM, one wait over all
- * groups, one consumer launch: nothing that short can hide a fork and a join);
+ * keeps the whole call on the GEMM stream (the GEMM with its reordered store,
+ * then one consumer launch: nothing that short can hide a fork and a join, and
+ * the stream orders the two, so MM is not touched and stays zero; with the
+ * monitor on, the signalling GEMM and one wait over all groups as elsewhere);
  * otherwise one launch when there are more than 16 groups, else per-wave
  * launches.  0: always the second stream with wait + consumer launches per
  * group (per GEMM wave) as the reference's host loop

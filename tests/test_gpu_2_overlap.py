@@ -69,6 +69,42 @@ def test_allreduce_overlap_against_checker(fo, oracle, dtype, fused):
     ov.close()
 
 
+def test_short_gemm_on_one_stream_with_and_without_monitor(fo):
+    # automatic mode keeps a GEMM this short on one stream; without the monitor it then
+    # leaves the counters alone, with it the stamps are written and the waits reset the groups
+    bm, bn, M, N, K = 128, 128, 1024, 1024, 128
+    cseg = [16, 16, 8, 24]
+    algo, RA, A, B, _, _, MM, cs_cpu, cs_gpu = _setup(fo, F16, bm, bn, M, N, K, cseg)
+    TM, TN = RA.shape
+    T = TM * TN
+    ov = fo.ops.Overlap()
+    ACC = torch.zeros(M * N, device="cuda", dtype=torch.float16)
+    ov.set_accumulator(ACC)
+    quiet = torch.empty(M * N, device="cuda", dtype=torch.float16)
+    ov.gemm_allreduce_overlap(A, B, quiet, MM, RA, 1, cs_cpu, cs_gpu, algo)
+    torch.cuda.synchronize()
+    assert (MM == 0).all()
+    assert torch.equal(ACC, quiet)
+    stamped = torch.empty_like(quiet)
+    MMm = torch.zeros(fo.layout.counter_size(len(cseg), TM, TN, monitor=True), dtype=torch.int32, device="cuda")
+    ov.gemm_allreduce_overlap(A, B, stamped, MMm, RA, 1, cs_cpu, cs_gpu, algo, monitor=True)
+    torch.cuda.synchronize()
+    mm = MMm.cpu()
+    assert (mm[:len(cseg)] == 0).all()                       # reset by the wait
+    assert mm[TN - 1].item() == T                            # completion counter
+    assert sorted(mm[TN:TN + T].tolist()) == list(range(T))  # one stamp per tile
+    assert torch.equal(stamped, quiet)
+    # forced onto two streams: same tiles, same accumulation
+    MM.zero_()
+    ACC.zero_()
+    ov.set_fused_consumer(0)
+    two = torch.empty_like(quiet)
+    ov.gemm_allreduce_overlap(A, B, two, MM, RA, 1, cs_cpu, cs_gpu, algo)
+    torch.cuda.synchronize()
+    assert torch.equal(two, quiet) and torch.equal(ACC, quiet) and (MM == 0).all()
+    ov.close()
+
+
 @pytest.mark.parametrize("fused", [False, True, -1])
 def test_reducescatter_overlap_segments(fo, oracle, fused):
     dtype, W, rank = F16, 4, 2
