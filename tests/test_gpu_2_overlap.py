@@ -459,6 +459,39 @@ def test_uneven_tile_walk_matches_vendor_gemm(fo):
     assert torch.equal(fo.layout.unpermute(Cp, M, N, bm, bn, RA), C)
 
 
+@pytest.mark.parametrize("fused", [0, 1, -1])
+def test_overlap_with_a_partial_last_wave(fo, fused):
+    """320 workgroup tiles: one full wave of 256, then 64 positions that a second GEMM launch computes
+    in 128x128 tiles.  The overlapped call must still hand every group to the consumer exactly once."""
+    M, N, K, bm, bn = 4096, 5120, 256, 128, 128
+    algo = fo._capi.find_algo(bm, bn, swizzle=4)
+    TM, TN = M // bm, N // bn
+    T = TM * TN
+    cseg = [512, 512, 256]
+    assert sum(cseg) == T
+    g = torch.Generator(device="cuda").manual_seed(77)
+    A = torch.randn(M, K, device="cuda", generator=g).half()
+    B = (torch.randn(N, K, device="cuda", generator=g) * K ** -0.5).half()
+    RA = fo.layout.reorder_indices(T, fo._capi.schedule_order(algo, M, N), device="cuda").reshape(TM, TN)
+    MM = torch.zeros(fo.layout.counter_size(len(cseg), TM, TN), dtype=torch.int32, device="cuda")
+    cs_cpu = torch.tensor(cseg, dtype=torch.int32)
+    C = torch.empty(M, N, device="cuda", dtype=torch.float16)
+    fo.ops.gemm(A, B, C, algo)
+    Cp = torch.full((M * N,), float("nan"), device="cuda", dtype=torch.float16)
+    ACC = torch.zeros(M * N, device="cuda", dtype=torch.float16)
+    ov = fo.ops.Overlap()
+    ov.set_fused_consumer(fused)
+    ov.set_accumulator(ACC)
+    for _ in range(2):
+        ov.gemm_allreduce_overlap(A, B, Cp, MM, RA, 1, cs_cpu, cs_cpu.cuda(), algo)
+    torch.cuda.synchronize()
+    assert (MM == 0).all()
+    assert torch.equal(fo.layout.unpermute(Cp, M, N, bm, bn, RA), C)
+    twice = (C.float() * 2).half()                       # 0 + c, then c + c: both sums are exact
+    assert torch.equal(fo.layout.unpermute(ACC, M, N, bm, bn, RA), twice)
+    ov.close()
+
+
 @pytest.mark.parametrize("fused", [0, 1])
 def test_overlapped_step_captured_in_a_hip_graph(fo, fused):
     """Capture {overlapped GEMM + consumer, reorder+RMSNorm} once, replay it several times with eager
