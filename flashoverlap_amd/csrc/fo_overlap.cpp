@@ -235,7 +235,7 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
                                          const int32_t *RA, int TM, int TN, int rLDN,
                                          const int32_t *cseg_host, const int32_t *cseg_dev, int G,
                                          int algo, int monitor) {
-    if (!h) return FO_ERR_ARG;
+    if (!h || !MM) return FO_ERR_ARG;
     if (!h->gemm_ready || !h->overlap_ready) return FO_ERR_STATE;
     int32_t info[12];
     int rc = fo_algo_info(algo, info);
@@ -266,7 +266,6 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
     // to do: unless the caller wants the monitor's stamps, the GEMM then leaves
     // the counters alone (they stay zero, as the waits would have left them).
     const bool quiet = same_stream && !monitor;
-    if (!MM) return FO_ERR_ARG;
     rc = quiet ? fo_gemm_reordered_quiet(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, RA, nullptr, algo,
                                          h->gemm_stream)
                : fo_gemm_signal(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, MM, RA, monitor, algo,
@@ -310,7 +309,7 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
                                              int32_t *MM, const int32_t *RA, const int32_t *RE,
                                              int TM, int TN, int rLDN, const int32_t *cseg_host,
                                              const int32_t *cseg_dev, int G, int algo, int monitor) {
-    if (!h) return FO_ERR_ARG;
+    if (!h || !MM || !RE) return FO_ERR_ARG;
     if (!h->gemm_ready || !h->overlap_ready) return FO_ERR_STATE;
     int32_t info[12];
     int rc = fo_algo_info(algo, info);
@@ -341,7 +340,6 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
         if (rc) return rc;
     }
     const bool quiet = same_stream && !monitor;  // as in fo_overlap_gemm_allreduce
-    if (!MM || !RE) return FO_ERR_ARG;
     rc = quiet ? fo_gemm_reordered_quiet(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, RA, RE, algo,
                                          h->gemm_stream)
                : fo_gemm_scatter(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, MM, RA, RE, monitor, algo,
