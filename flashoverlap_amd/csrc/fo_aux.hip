@@ -101,7 +101,12 @@ __device__ __forceinline__ fo_u32x4 load16_coherent(const fo_u32x4 *base, unsign
 // With `own` set, the pieces of chunk `rank` are also copied to own + (i - rank*chunk16): this
 // rank's share of the group, the output of a reduce-scatter with one rank present.
 // COHERENT: src is read past the caches (see load16_coherent).
-template <typename Tag, bool RS, bool COHERENT>
+// STREAM: dst is read and written with non-temporal accesses.  An accumulator that is touched
+// once per step and does not fit into the 256 MB memory-side cache beside everything else
+// only evicts what will be used again (the GEMM's operands, the tiles the RMSNorm reads next):
+// measured inside the overlapped step, 8192x8192 outputs, -2 % (K = 8192) and -9 % (K = 3584)
+// of the whole step; on a 67 MB accumulator that is read again right away it costs 2 %.
+template <typename Tag, bool RS, bool COHERENT, bool STREAM>
 __device__ __forceinline__ void reduce_range(const fo_u32x4 *src, fo_u32x4 *dst, long lo, long hi,
                                              long chunk16, long seg_stride16, int tid, int nthreads,
                                              fo_u32x4 *own = nullptr, int rank = 0) {
@@ -129,9 +134,19 @@ __device__ __forceinline__ void reduce_range(const fo_u32x4 *src, fo_u32x4 *dst,
 #pragma unroll
         for (int u = 0; u < U; u++) a[u] = fetch(first, u);
 #pragma unroll
-        for (int u = 0; u < U; u++) b[u] = *where(i + (long)u * nthreads);
+        for (int u = 0; u < U; u++) {
+            fo_u32x4 *d = where(i + (long)u * nthreads);
+            b[u] = STREAM ? __builtin_nontemporal_load(d) : *d;
+        }
 #pragma unroll
-        for (int u = 0; u < U; u++) *where(i + (long)u * nthreads) = add8<Tag>(b[u], a[u]);
+        for (int u = 0; u < U; u++) {
+            fo_u32x4 *d = where(i + (long)u * nthreads);
+            const fo_u32x4 v = add8<Tag>(b[u], a[u]);
+            if (STREAM)
+                __builtin_nontemporal_store(v, d);
+            else
+                *d = v;
+        }
 #pragma unroll
         for (int u = 0; u < U; u++) keep(i + (long)u * nthreads, a[u]);
     }
@@ -139,7 +154,11 @@ __device__ __forceinline__ void reduce_range(const fo_u32x4 *src, fo_u32x4 *dst,
         if (first + tid < hi) {
             fo_u32x4 *d = where(first + tid);
             const fo_u32x4 a = fetch(first, 0);
-            *d = add8<Tag>(*d, a);
+            const fo_u32x4 v = add8<Tag>(STREAM ? __builtin_nontemporal_load(d) : *d, a);
+            if (STREAM)
+                __builtin_nontemporal_store(v, d);
+            else
+                *d = v;
             keep(first + tid, a);
         }
     }
@@ -150,17 +169,24 @@ template <typename Tag>
 __global__ __launch_bounds__(CONSUMER_THREADS, 8) void fo_consumer_kernel(const fo_u32x4 *src, fo_u32x4 *acc,
                                                                        long chunk16, int W,
                                                                        long seg_stride16, fo_u32x4 *own,
-                                                                       int rank) {
+                                                                       int rank, int stream_acc) {
     const long total = chunk16 * W;
     const long per = (total + gridDim.x - 1) / gridDim.x;
     const long lo = per * blockIdx.x;
     const long hi = lo + per < total ? lo + per : total;
     if (lo >= hi) return;
-    if (W <= 1)
-        reduce_range<Tag, false, false>(src, acc, lo, hi, 0, 0, threadIdx.x, blockDim.x);
-    else
-        reduce_range<Tag, true, false>(src, acc, lo, hi, chunk16, seg_stride16, threadIdx.x, blockDim.x, own,
-                                       rank);
+    if (W <= 1) {
+        if (stream_acc)
+            reduce_range<Tag, false, false, true>(src, acc, lo, hi, 0, 0, threadIdx.x, blockDim.x);
+        else
+            reduce_range<Tag, false, false, false>(src, acc, lo, hi, 0, 0, threadIdx.x, blockDim.x);
+    } else if (stream_acc) {
+        reduce_range<Tag, true, false, true>(src, acc, lo, hi, chunk16, seg_stride16, threadIdx.x, blockDim.x, own,
+                                             rank);
+    } else {
+        reduce_range<Tag, true, false, false>(src, acc, lo, hi, chunk16, seg_stride16, threadIdx.x, blockDim.x, own,
+                                              rank);
+    }
 }
 
 // The same for `ngroups` consecutive groups in one launch (blockIdx.y = group):
@@ -170,7 +196,7 @@ __global__ __launch_bounds__(CONSUMER_THREADS, 8) void fo_consumer_kernel(const 
 template <typename Tag>
 __global__ __launch_bounds__(CONSUMER_THREADS, 8) void fo_consumer_groups_kernel(
     const fo_u32x4 *src, fo_u32x4 *acc, const int32_t *cseg, long tile16, int W, long seg_stride16,
-    fo_u32x4 *own, int rank) {
+    fo_u32x4 *own, int rank, int stream_acc) {
     long off = 0;
     for (int k = 0; k < (int)blockIdx.y; k++) off += cseg[k];
     off *= tile16;
@@ -179,8 +205,12 @@ __global__ __launch_bounds__(CONSUMER_THREADS, 8) void fo_consumer_groups_kernel
     const long lo = per * blockIdx.x;
     const long hi = lo + per < total ? lo + per : total;
     if (lo >= hi) return;
-    reduce_range<Tag, true, false>(src + off, acc + off / W, lo, hi, total / W, seg_stride16, threadIdx.x,
-                                   blockDim.x, own ? own + off / W : nullptr, rank);
+    if (stream_acc)
+        reduce_range<Tag, true, false, true>(src + off, acc + off / W, lo, hi, total / W, seg_stride16, threadIdx.x,
+                                             blockDim.x, own ? own + off / W : nullptr, rank);
+    else
+        reduce_range<Tag, true, false, false>(src + off, acc + off / W, lo, hi, total / W, seg_stride16,
+                                              threadIdx.x, blockDim.x, own ? own + off / W : nullptr, rank);
 }
 
 // One launch for all groups.  The work is cut into items (group g, slice s of
@@ -209,7 +239,8 @@ __global__ __launch_bounds__(CONSUMER_THREADS, 8) void fo_consumer_groups_kernel
 template <typename Tag>
 __global__ __launch_bounds__(CONSUMER_THREADS, 8) void fo_wait_reduce_kernel(
     const fo_u32x4 *C, fo_u32x4 *ACC, int32_t *MM, const int32_t *cseg, int G, long tile16, int W,
-    long seg_stride16, int slices, int32_t *ws, long max_polls, int sleep_ticks, fo_u32x4 *OWN, int rank) {
+    long seg_stride16, int slices, int32_t *ws, long max_polls, int sleep_ticks, fo_u32x4 *OWN, int rank,
+    int stream_acc) {
     __shared__ int first_tile_s, last;
     const int nb = gridDim.x;
     const long items = (long)G * slices;
@@ -237,11 +268,21 @@ __global__ __launch_bounds__(CONSUMER_THREADS, 8) void fo_wait_reduce_kernel(
             const long base16 = (long)first_tile_s * tile16;
             const long n16 = (long)cnt * tile16;
             const long lo = n16 * sl / slices, hi = n16 * (sl + 1) / slices;
-            if (W <= 1)
-                reduce_range<Tag, false, true>(C + base16, ACC + base16, lo, hi, 0, 0, threadIdx.x, blockDim.x);
-            else
-                reduce_range<Tag, true, true>(C + base16, ACC + base16 / W, lo, hi, n16 / W, seg_stride16,
-                                              threadIdx.x, blockDim.x, OWN ? OWN + base16 / W : nullptr, rank);
+            fo_u32x4 *own = OWN ? OWN + base16 / W : nullptr;
+            if (W <= 1) {
+                if (stream_acc)
+                    reduce_range<Tag, false, true, true>(C + base16, ACC + base16, lo, hi, 0, 0, threadIdx.x,
+                                                         blockDim.x);
+                else
+                    reduce_range<Tag, false, true, false>(C + base16, ACC + base16, lo, hi, 0, 0, threadIdx.x,
+                                                          blockDim.x);
+            } else if (stream_acc) {
+                reduce_range<Tag, true, true, true>(C + base16, ACC + base16 / W, lo, hi, n16 / W, seg_stride16,
+                                                    threadIdx.x, blockDim.x, own, rank);
+            } else {
+                reduce_range<Tag, true, true, false>(C + base16, ACC + base16 / W, lo, hi, n16 / W, seg_stride16,
+                                                     threadIdx.x, blockDim.x, own, rank);
+            }
         }
         __syncthreads();  // first_tile_s is rewritten for the next item
     }
@@ -264,7 +305,10 @@ __global__ __launch_bounds__(CONSUMER_THREADS, 8) void fo_wait_reduce_kernel(
 // from the tile-reordered buffer (index math of src/rmsnorm/rmsnorm.cuh:80-86).
 // The second launch bound caps the registers (128 up to 16 chunks per lane, 256 above) so that
 // enough wavefronts stay resident to cover the memory latency.
-template <typename Tag, int MAXCH>
+// STREAM: rows are read and written with non-temporal accesses (matrices that do not fit
+// into the memory-side cache beside the GEMM's operands: inside the overlapped step the
+// 8192x8192 RMSNorm then takes 55 instead of 64 us, and the GEMM that follows it 3 % less).
+template <typename Tag, int MAXCH, bool STREAM>
 __global__ __launch_bounds__(256, MAXCH <= 16 ? 4 : 2) void fo_rmsnorm_kernel(const fo_u32x4 *X, fo_u32x4 *Y, const fo_u32x4 *Wt,
                                                          int bs, int dim, int BM, int BN, int rldn,
                                                          const int32_t *RA, float eps) {
@@ -301,7 +345,7 @@ __global__ __launch_bounds__(256, MAXCH <= 16 ? 4 : 2) void fo_rmsnorm_kernel(co
             } else {
                 src = (long)b * nch + c;
             }
-            x[i] = X[src];
+            x[i] = STREAM ? __builtin_nontemporal_load(&X[src]) : X[src];
             const uint32_t w[4] = {x[i].x, x[i].y, x[i].z, x[i].w};
 #pragma unroll
             for (int k = 0; k < 4; k++) {
@@ -335,31 +379,44 @@ __global__ __launch_bounds__(256, MAXCH <= 16 ? 4 : 2) void fo_rmsnorm_kernel(co
                 const uint16_t yhi = E::from_f32(hi * E::to_f32((uint16_t)(wi[k] >> 16)));
                 o[k] = (uint32_t)ylo | ((uint32_t)yhi << 16);
             }
-            Y[(long)b * nch + c] = fo_u32x4{o[0], o[1], o[2], o[3]};
+            const fo_u32x4 y = {o[0], o[1], o[2], o[3]};
+            if (STREAM)
+                __builtin_nontemporal_store(y, &Y[(long)b * nch + c]);
+            else
+                Y[(long)b * nch + c] = y;
         }
     }
 }
 
-template <typename Tag>
-int launch_rmsnorm(const void *X, void *Y, const void *Wt, int bs, int dim, int BM, int BN,
-                   int rldn, const int32_t *RA, float eps, hipStream_t stream) {
+template <typename Tag, bool STREAM>
+int launch_rmsnorm_as(const void *X, void *Y, const void *Wt, int bs, int dim, int BM, int BN,
+                      int rldn, const int32_t *RA, float eps, hipStream_t stream) {
     const int nch = dim / 8;
     dim3 grid((bs + 3) / 4), block(256);
     const fo_u32x4 *x = static_cast<const fo_u32x4 *>(X);
     fo_u32x4 *y = static_cast<fo_u32x4 *>(Y);
     const fo_u32x4 *w = static_cast<const fo_u32x4 *>(Wt);
     if (nch <= 64 * 4)
-        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 4>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
+        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 4, STREAM>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
     else if (nch <= 64 * 8)
-        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 8>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
+        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 8, STREAM>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
     else if (nch <= 64 * 16)
-        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 16>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
+        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 16, STREAM>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
     else if (nch <= 64 * 32)
-        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 32>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
+        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 32, STREAM>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
     else
         return FO_ERR_SHAPE;  // rows above 16384 elements (the reference's limit too)
     FO_LAUNCH_CHECK();
     return FO_OK;
+}
+
+template <typename Tag>
+int launch_rmsnorm(const void *X, void *Y, const void *Wt, int bs, int dim, int BM, int BN,
+                   int rldn, const int32_t *RA, float eps, hipStream_t stream) {
+    // input and output together against the cache that would have to hold them
+    if (fo_streams((int64_t)bs * dim * 4))
+        return launch_rmsnorm_as<Tag, true>(X, Y, Wt, bs, dim, BM, BN, rldn, RA, eps, stream);
+    return launch_rmsnorm_as<Tag, false>(X, Y, Wt, bs, dim, BM, BN, rldn, RA, eps, stream);
 }
 
 // FO_WAIT_MAX_POLLS (environment, read once): bound for the otherwise unbounded
@@ -416,8 +473,8 @@ extern "C" int fo_wait_bounded(int expect, int32_t *counter, int64_t max_polls, 
     return FO_OK;
 }
 
-extern "C" int fo_consumer_reduce_rs_own(int dtype, const void *src, void *acc, int64_t nelem, int W,
-                                         int64_t seg_stride, void *own, int rank, fo_stream_t stream) {
+int fo_consumer_reduce_with(int dtype, const void *src, void *acc, int64_t nelem, int W, int64_t seg_stride,
+                            void *own, int rank, bool stream_acc, fo_stream_t stream) {
     if (!src || !acc || nelem < 0 || W <= 0) return FO_ERR_ARG;
     if (own && (rank < 0 || rank >= W)) return FO_ERR_ARG;
     if (nelem == 0) return FO_OK;
@@ -433,19 +490,29 @@ extern "C" int fo_consumer_reduce_rs_own(int dtype, const void *src, void *acc, 
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == FO_F16)
         hipLaunchKernelGGL(fo_consumer_kernel<fo_f16_tag>, grid, block, 0, s, (const fo_u32x4 *)src,
-                           (fo_u32x4 *)acc, chunk16, W, (long)(seg_stride / 8), (fo_u32x4 *)own, rank);
+                           (fo_u32x4 *)acc, chunk16, W, (long)(seg_stride / 8), (fo_u32x4 *)own, rank,
+                           (int)stream_acc);
     else if (dtype == FO_BF16)
         hipLaunchKernelGGL(fo_consumer_kernel<fo_bf16_tag>, grid, block, 0, s, (const fo_u32x4 *)src,
-                           (fo_u32x4 *)acc, chunk16, W, (long)(seg_stride / 8), (fo_u32x4 *)own, rank);
+                           (fo_u32x4 *)acc, chunk16, W, (long)(seg_stride / 8), (fo_u32x4 *)own, rank,
+                           (int)stream_acc);
     else
         return FO_ERR_DTYPE;
     FO_LAUNCH_CHECK();
     return FO_OK;
 }
 
-extern "C" int fo_consumer_reduce_rs_groups(int dtype, const void *src, void *acc, const int32_t *cseg_dev,
-                                            int ngroups, int64_t max_group_tiles, int64_t tile_elems, int W,
-                                            int64_t seg_stride, void *own, int rank, fo_stream_t stream) {
+// The entry points below know only their own range: source and accumulator
+// together decide.  The overlapped calls, which know the whole matrix, use the
+// *_with forms.
+extern "C" int fo_consumer_reduce_rs_own(int dtype, const void *src, void *acc, int64_t nelem, int W,
+                                         int64_t seg_stride, void *own, int rank, fo_stream_t stream) {
+    return fo_consumer_reduce_with(dtype, src, acc, nelem, W, seg_stride, own, rank, fo_streams(nelem * 4), stream);
+}
+
+int fo_consumer_reduce_groups_with(int dtype, const void *src, void *acc, const int32_t *cseg_dev, int ngroups,
+                                   int64_t max_group_tiles, int64_t tile_elems, int W, int64_t seg_stride,
+                                   void *own, int rank, bool stream_acc, fo_stream_t stream) {
     if (!src || !acc || !cseg_dev || ngroups <= 0 || max_group_tiles <= 0 || tile_elems <= 0 || W < 2)
         return FO_ERR_ARG;
     if (own && (rank < 0 || rank >= W)) return FO_ERR_ARG;
@@ -459,14 +526,24 @@ extern "C" int fo_consumer_reduce_rs_groups(int dtype, const void *src, void *ac
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == FO_F16)
         hipLaunchKernelGGL(fo_consumer_groups_kernel<fo_f16_tag>, grid, block, 0, s, (const fo_u32x4 *)src,
-                           (fo_u32x4 *)acc, cseg_dev, tile16, W, (long)(seg_stride / 8), (fo_u32x4 *)own, rank);
+                           (fo_u32x4 *)acc, cseg_dev, tile16, W, (long)(seg_stride / 8), (fo_u32x4 *)own, rank,
+                           (int)stream_acc);
     else if (dtype == FO_BF16)
         hipLaunchKernelGGL(fo_consumer_groups_kernel<fo_bf16_tag>, grid, block, 0, s, (const fo_u32x4 *)src,
-                           (fo_u32x4 *)acc, cseg_dev, tile16, W, (long)(seg_stride / 8), (fo_u32x4 *)own, rank);
+                           (fo_u32x4 *)acc, cseg_dev, tile16, W, (long)(seg_stride / 8), (fo_u32x4 *)own, rank,
+                           (int)stream_acc);
     else
         return FO_ERR_DTYPE;
     FO_LAUNCH_CHECK();
     return FO_OK;
+}
+
+extern "C" int fo_consumer_reduce_rs_groups(int dtype, const void *src, void *acc, const int32_t *cseg_dev,
+                                            int ngroups, int64_t max_group_tiles, int64_t tile_elems, int W,
+                                            int64_t seg_stride, void *own, int rank, fo_stream_t stream) {
+    return fo_consumer_reduce_groups_with(dtype, src, acc, cseg_dev, ngroups, max_group_tiles, tile_elems, W,
+                                          seg_stride, own, rank,
+                                          fo_streams(max_group_tiles * tile_elems * ngroups * 4), stream);
 }
 
 extern "C" int fo_consumer_reduce_rs(int dtype, const void *src, void *acc, int64_t nelem, int W,
@@ -479,10 +556,10 @@ extern "C" int fo_consumer_reduce(int dtype, const void *src, void *acc, int64_t
     return fo_consumer_reduce_rs(dtype, src, acc, nelem, 1, 0, stream);
 }
 
-extern "C" int fo_wait_reduce_groups(int dtype, const void *C, void *ACC, int32_t *MM,
-                                     const int32_t *cseg_dev, int G, int64_t tile_elems, int W,
-                                     int64_t seg_stride, void *own, int rank, int32_t *workspace,
-                                     int nblocks, int slices, int poll_gap_ns, fo_stream_t stream) {
+int fo_wait_reduce_groups_with(int dtype, const void *C, void *ACC, int32_t *MM, const int32_t *cseg_dev, int G,
+                               int64_t tile_elems, int W, int64_t seg_stride, void *own, int rank,
+                               int32_t *workspace, int nblocks, int slices, int poll_gap_ns, bool stream_acc,
+                               fo_stream_t stream) {
     if (!MM || !cseg_dev || !workspace || G <= 0 || tile_elems <= 0 || W <= 0) return FO_ERR_ARG;
     if (ACC && !C) return FO_ERR_ARG;
     if (own && (!ACC || W < 2 || rank < 0 || rank >= W)) return FO_ERR_ARG;
@@ -503,16 +580,26 @@ extern "C" int fo_wait_reduce_groups(int dtype, const void *C, void *ACC, int32_
         hipLaunchKernelGGL(fo_wait_reduce_kernel<fo_f16_tag>, grid, block, 0, s, (const fo_u32x4 *)C,
                            (fo_u32x4 *)ACC, MM, cseg_dev, G, (long)(tile_elems / 8), W,
                            (long)(seg_stride / 8), slices, workspace, default_max_polls(), sleep_ticks,
-                           (fo_u32x4 *)own, rank);
+                           (fo_u32x4 *)own, rank, (int)stream_acc);
     else if (dtype == FO_BF16)
         hipLaunchKernelGGL(fo_wait_reduce_kernel<fo_bf16_tag>, grid, block, 0, s, (const fo_u32x4 *)C,
                            (fo_u32x4 *)ACC, MM, cseg_dev, G, (long)(tile_elems / 8), W,
                            (long)(seg_stride / 8), slices, workspace, default_max_polls(), sleep_ticks,
-                           (fo_u32x4 *)own, rank);
+                           (fo_u32x4 *)own, rank, (int)stream_acc);
     else
         return FO_ERR_DTYPE;
     FO_LAUNCH_CHECK();
     return FO_OK;
+}
+
+// The group sizes live on the device: without the whole matrix's size the
+// accumulator is treated as cacheable.
+extern "C" int fo_wait_reduce_groups(int dtype, const void *C, void *ACC, int32_t *MM,
+                                     const int32_t *cseg_dev, int G, int64_t tile_elems, int W,
+                                     int64_t seg_stride, void *own, int rank, int32_t *workspace,
+                                     int nblocks, int slices, int poll_gap_ns, fo_stream_t stream) {
+    return fo_wait_reduce_groups_with(dtype, C, ACC, MM, cseg_dev, G, tile_elems, W, seg_stride, own, rank,
+                                      workspace, nblocks, slices, poll_gap_ns, false, stream);
 }
 
 extern "C" int fo_reorder_rmsnorm(int dtype, const void *X, void *Y, const void *Wt, int bs, int dim,

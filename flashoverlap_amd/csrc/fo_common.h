@@ -101,6 +101,24 @@ int fo_gemm_reordered_quiet(int dtype, int M, int N, int K, int rLDN, const int3
                             const void *A, const void *B, void *C, const int32_t *RA, const int32_t *RE,
                             int algo, fo_stream_t stream);
 
+// Data that is touched once per step is moved with non-temporal accesses when the
+// step's working set cannot stay in the 256 MB memory-side cache anyway; below
+// that it is left cacheable, because the next kernel reads it again.
+constexpr int64_t kStreamAboveBytes = 192LL << 20;
+inline bool fo_streams(int64_t bytes) { return bytes > kStreamAboveBytes; }
+
+// The consumer entry points with the accumulator's cache policy chosen by the
+// caller (fo_aux.hip; the extern "C" forms decide from their own range).
+int fo_consumer_reduce_with(int dtype, const void *src, void *acc, int64_t nelem, int W, int64_t seg_stride,
+                            void *own, int rank, bool stream_acc, fo_stream_t stream);
+int fo_consumer_reduce_groups_with(int dtype, const void *src, void *acc, const int32_t *cseg_dev, int ngroups,
+                                   int64_t max_group_tiles, int64_t tile_elems, int W, int64_t seg_stride,
+                                   void *own, int rank, bool stream_acc, fo_stream_t stream);
+int fo_wait_reduce_groups_with(int dtype, const void *C, void *ACC, int32_t *MM, const int32_t *cseg_dev, int G,
+                               int64_t tile_elems, int W, int64_t seg_stride, void *own, int rank,
+                               int32_t *workspace, int nblocks, int slices, int poll_gap_ns, bool stream_acc,
+                               fo_stream_t stream);
+
 // Workgroup id -> macro tile coordinates; identical code on host and device.
 __host__ __device__ inline void fo_wg_to_tile(int wg, int grid_m, int grid_n, int panel,
                                               int xcd_remap, int *pm, int *pn) {

@@ -272,10 +272,12 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
                                 h->gemm_stream);
     if (rc) return rc;  // nothing has been enqueued on the consumer stream yet
 
+    // C' and the accumulator together against the memory-side cache
+    const bool stream_acc = fo_streams((int64_t)M * N * 4);
     if (fused) {
-        rc = fo_wait_reduce_groups(dtype, C, h->acc, MM, cseg_dev, G, tile_elems, 1, 0, nullptr, 0,
-                                   h->workspace, fused, fused_slices((int64_t)M * N, G, fused),
-                                   fused_poll_gap_ns(M, N, K, fused), h->comm_stream);
+        rc = fo_wait_reduce_groups_with(dtype, C, h->acc, MM, cseg_dev, G, tile_elems, 1, 0, nullptr, 0,
+                                        h->workspace, fused, fused_slices((int64_t)M * N, G, fused),
+                                        fused_poll_gap_ns(M, N, K, fused), stream_acc, h->comm_stream);
         if (rc) return rc;
     } else {
         int64_t off = 0;
@@ -293,7 +295,7 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
                 if (rc) return rc;
             }
             if (acc) {  // the groups of a batch are one contiguous range
-                rc = fo_consumer_reduce(dtype, c + off, acc + off, n, cstream);
+                rc = fo_consumer_reduce_with(dtype, c + off, acc + off, n, 1, 0, nullptr, 0, stream_acc, cstream);
                 if (rc) return rc;
             }
             off += n;
@@ -353,11 +355,12 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
     // every group to D (ncclReduceScatter(C+acc -> D+acc/W, n/W) with one rank
     // present, src/overlap_impl.cu:312-313); otherwise a copy per group does.
     const bool own_in_consumer = d && acc && W > 1;
+    const bool stream_acc = fo_streams((int64_t)M * N * 4);
     if (fused) {
-        rc = fo_wait_reduce_groups(dtype, C, h->acc, MM, cseg_dev, G, tile_elems, W, seg_stride,
-                                   own_in_consumer ? D : nullptr, h->rank, h->workspace, fused,
-                                   fused_slices((int64_t)M * N, G, fused), fused_poll_gap_ns(M, N, K, fused),
-                                   cstream);
+        rc = fo_wait_reduce_groups_with(dtype, C, h->acc, MM, cseg_dev, G, tile_elems, W, seg_stride,
+                                        own_in_consumer ? D : nullptr, h->rank, h->workspace, fused,
+                                        fused_slices((int64_t)M * N, G, fused), fused_poll_gap_ns(M, N, K, fused),
+                                        stream_acc, cstream);
         if (rc) return rc;
     }
     int64_t off = 0;
@@ -373,16 +376,16 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
             // the groups of one wave in one launch; each keeps its own W chunks
             long most = 0;
             for (int g = i; g < j; g++) most = cseg_host[g] > most ? cseg_host[g] : most;
-            rc = fo_consumer_reduce_rs_groups(dtype, c + off, acc + off / W, cseg_dev + i, j - i, most, tile_elems,
-                                              W, seg_stride, own_in_consumer ? d + off / W : nullptr, h->rank,
-                                              cstream);
+            rc = fo_consumer_reduce_groups_with(dtype, c + off, acc + off / W, cseg_dev + i, j - i, most,
+                                                tile_elems, W, seg_stride, own_in_consumer ? d + off / W : nullptr,
+                                                h->rank, stream_acc, cstream);
             if (rc) return rc;
         }
         for (int g = i; g < j; g++) {
             const int64_t n = cseg_host[g] * tile_elems;
             if (!fused && acc && !(W > 1 && j - i > 1)) {
-                rc = fo_consumer_reduce_rs_own(dtype, c + off, acc + off / W, n, W, seg_stride,
-                                               own_in_consumer ? d + off / W : nullptr, h->rank, cstream);
+                rc = fo_consumer_reduce_with(dtype, c + off, acc + off / W, n, W, seg_stride,
+                                             own_in_consumer ? d + off / W : nullptr, h->rank, stream_acc, cstream);
                 if (rc) return rc;
             }
             if (d && !own_in_consumer)
