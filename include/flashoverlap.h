@@ -137,7 +137,13 @@ int fo_wait_bounded(int expect, int32_t *counter, int64_t max_polls, int32_t *st
 /* ---- consumer (1-GPU stand-in for the collective) ------------------------
  * Stands in for ncclAllReduce(C+acc, C+acc, n, half, sum) at
  * src/overlap_impl.cu:256: acc[i] = round(float(acc[i]) + float(src[i])),
- * i < nelem; nelem % 8 == 0, 16-byte aligned pointers. */
+ * i < nelem; nelem % 8 == 0, 16-byte aligned pointers.
+ * Cache policy (no effect on results): when source and accumulator together
+ * exceed 192 MB the accumulator is read and written with non-temporal
+ * accesses, so that it does not evict reusable data from the 256 MB
+ * memory-side cache; the overlapped calls decide this from M*N instead of
+ * the single range.  fo_reorder_rmsnorm / fo_rmsnorm do the same with their
+ * rows (input + output above 192 MB). */
 int fo_consumer_reduce(int dtype, const void *src, void *acc, int64_t nelem, fo_stream_t stream);
 
 /* Stands in for ncclReduceScatter(C+acc, D+acc/W, n/W) at
