@@ -322,18 +322,39 @@ __global__ __launch_bounds__(256, MAXCH <= 16 ? 4 : 2) void fo_rmsnorm_kernel(co
     const long ldp16 = RA ? ((long)rldn * BN) >> 3 : 0;
     const int bn_shift = (RA && rldn == 1 && (BN & (BN - 1)) == 0) ? __builtin_ctz(BN) : -1;
 
+    // The storage slots of this row's tiles, fetched once per wavefront (lane l holds the
+    // slots of tiles l and l + 64) and handed out by shuffles: a table load per chunk would
+    // put a second memory round trip in front of every load of the row (measured with
+    // nothing cached, 8192 x 8192: 69 us against 52 us for the plain RMSNorm).
+    const bool slots_in_lanes = bn_shift >= 0 && ldn <= 128;
+    int slot_lo = 0, slot_hi = 0;
+    if (slots_in_lanes) {
+        const int32_t *row = RA + (long)tile_row * ldn;
+        if (lane < ldn) slot_lo = row[lane];
+        if (lane + 64 < ldn) slot_hi = row[lane + 64];
+    }
+
     fo_u32x4 x[MAXCH];
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < MAXCH; i++) {
         const int c = lane + i * 64;
+        // shuffles are executed by all lanes; chunks beyond the row ask for tile 0
+        int r_lanes = 0;
+        if (slots_in_lanes) {
+            const int t = c < nch ? (c << 3) >> bn_shift : 0;
+            const int lo = __shfl(slot_lo, t & 63, 64), hi = __shfl(slot_hi, t & 63, 64);
+            r_lanes = t < 64 ? lo : hi;
+        }
         if (c < nch) {
             long src;
             if (RA) {
                 const int j = c << 3;
-                if (bn_shift >= 0) {
+                if (slots_in_lanes) {
                     // rldn == 1 and BN a power of two (every tile of the Algo table): tile r is
                     // the contiguous block of BM rows of BN columns that starts at row r * BM
+                    src = ((long)r_lanes * BM + in_row) * ldp16 + ((j & (BN - 1)) >> 3);
+                } else if (bn_shift >= 0) {
                     const int r = RA[tile_row * ldn + (j >> bn_shift)];
                     src = ((long)r * BM + in_row) * ldp16 + ((j & (BN - 1)) >> 3);
                 } else {
