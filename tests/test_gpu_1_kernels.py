@@ -286,6 +286,44 @@ def test_rmsnorm_constant_row_closed_form(fo):
 
 
 @pytest.mark.parametrize("dtype", [F16, BF16])
+def test_streaming_forms_give_the_same_bits(fo, dtype):
+    """Above 192 MB of footprint the consumer's accumulator and the RMSNorm's rows move with
+    non-temporal accesses: the values must be those of the cacheable forms that small inputs use."""
+    td = TORCH_DTYPE[dtype]
+    M = N = 8192                                             # 268 MB per kernel: streaming
+    g = torch.Generator(device="cuda").manual_seed(91)
+    src = torch.randn(M * N, device="cuda", generator=g).to(td)
+    acc = torch.randn(M * N, device="cuda", generator=g).to(td)
+    small = 1 << 20                                          # 4 MB: cacheable
+    ref_small = acc[:small].clone()
+    fo.ops.consumer_reduce(src[:small], ref_small)
+    expect = (acc.float() + src.float()).to(td)              # one rounding of the fp32 sum
+    fo.ops.consumer_reduce(src, acc)
+    torch.cuda.synchronize()
+    assert torch.equal(acc, expect)
+    assert torch.equal(acc[:small], ref_small)
+    # reorder+RMSNorm: the first tile row of the large run against a run on that tile row alone
+    bm, bn = 128, 256
+    TM, TN = M // bm, N // bn
+    ra = torch.randperm(TN, generator=torch.Generator().manual_seed(92)).to(torch.int32)
+    RA = (torch.arange(TM, dtype=torch.int32)[:, None] * TN + ra[None, :]).cuda()   # rows of tiles stay together
+    X = src.view(M, N)
+    Wt = (1 + 0.01 * torch.randn(N, device="cuda", generator=g)).to(td)
+    Y = torch.empty(M, N, device="cuda", dtype=td)
+    fo.ops.reorder_rmsnorm(X, Y, Wt, bm, bn, 1, RA, eps=1e-6)
+    Ys = torch.empty(bm, N, device="cuda", dtype=td)
+    fo.ops.reorder_rmsnorm(X[:bm], Ys, Wt, bm, bn, 1, RA[:1].contiguous(), eps=1e-6)
+    torch.cuda.synchronize()
+    assert torch.equal(Y[:bm], Ys)
+    Yp = torch.empty(M, N, device="cuda", dtype=td)
+    fo.ops.rmsnorm(X, Yp, Wt, eps=1e-6)
+    Yps = torch.empty(bm, N, device="cuda", dtype=td)
+    fo.ops.rmsnorm(X[:bm], Yps, Wt, eps=1e-6)
+    torch.cuda.synchronize()
+    assert torch.equal(Yp[:bm], Yps)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
 def test_reorder_rmsnorm_undoes_the_permutation(fo, oracle, dtype):
     for (bm, bn, M, N, rldn) in [(128, 128, 256, 1024, 1), (128, 256, 256, 4096, 1), (64, 128, 256, 512, 2),
                                  (16, 128, 64, 8192, 1), (32, 96, 64, 480, 1)]:  # last: BN no power of two
