@@ -7,6 +7,8 @@ headline metric is quoted on (fp16, M=N=K=8192, 128x256 tiles, wave groups of
 256 tiles).  Prints one JSON line; `value` is GEMM flops / step time.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c2|c3|c4] [--dtype f16|bf16]
+
+The default run (c5) appends compact records of the c2, c3 and c4 workloads as `other_workloads`.
 """
 import argparse
 import json
@@ -32,57 +34,21 @@ WORKLOADS = {
 }
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS))
-    ap.add_argument("--dtype", default=None, choices=["f16", "bf16"])
-    ap.add_argument("--swizzle", type=int, default=4)
-    ap.add_argument("--fused", type=int, default=-1,
-                    help="-1: library default (one wait+reduce launch above 16 groups), 0: two launches per "
-                         "group, 1: one launch")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--group-tiles", type=int, default=0, help="tiles per wave group (0: the workload's default)")
-    ap.add_argument("--no-group-sweep", action="store_true", help="skip the wave-group-size sweep (c5 only)")
-    ap.add_argument("--kernels-only", action="store_true",
-                    help="run each hot kernel alone on one stream and exit: for counter collection, which "
-                         "serialises dispatches and would stall a waiter that spins on another queue")
-    ap.add_argument("--steps-only", action="store_true",
-                    help="enqueue warmup + steps overlapped steps and exit: for a kernel-trace timeline of the "
-                         "steady state")
-    ap.add_argument("--copy-calibration", action="store_true",
-                    help="only run a 256 MiB device-to-device copy five times (reference point for "
-                         "scaling the FETCH_SIZE / WRITE_SIZE counters) and exit")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (the collective is "
-              "replaced by a one-GPU consumer); run with --gpus 1", file=sys.stderr)
-        sys.exit(2)
-
-    os.environ.setdefault("FO_WAIT_MAX_POLLS", "200000000")  # a lost signal must not hang the GPU
+def measure(args, workload, compact=False):
+    """Time one workload.  compact: the core figures only (the default run reports the other
+    BASELINE workloads this way, next to the full record of the headline one)."""
     import torch
     import flashoverlap_amd as fo
     from flashoverlap_amd import ops
 
-    torch.cuda.set_device(0)
-    if args.copy_calibration:
-        src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
-        dst = torch.empty_like(src)
-        for _ in range(5):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        print(json.dumps({"copy_bytes_read": src.numel(), "copy_bytes_written": dst.numel(), "copies": 5}))
-        return
-    M, N, K, BM, BN, dt, gtiles, W, desc = WORKLOADS[args.workload]
-    gtiles = args.group_tiles or gtiles
-    dt = args.dtype or dt
+    M, N, K, BM, BN, dt, gtiles, W, desc = WORKLOADS[workload]
+    gtiles = (args.group_tiles if not compact else 0) or gtiles
+    dt = (args.dtype if not compact else None) or dt
     td = torch.float16 if dt == "f16" else torch.bfloat16
     algo = fo._capi.find_algo(BM, BN, swizzle=args.swizzle)
     TM, TN = M // BM, N // BN
     T = TM * TN
-    if args.workload == "c3" and not args.group_tiles:
+    if workload == "c3" and (compact or not args.group_tiles):
         # wave-group sizes chosen by the predictive search (tune/search.py:442-502) from a measured
         # GEMM duration and the consumer's measured bandwidth curve
         from flashoverlap_amd import tune
@@ -100,12 +66,12 @@ def main():
     RE = fo.layout.generate_row_mapping(M, N, BM, BN, cseg, W, device="cuda") if W else None
 
     g = torch.Generator().manual_seed(0)
-    if args.workload == "c5":
+    if workload == "c5":
         A16 = ((torch.rand(M, K, generator=g) * 2 - 1) * K ** -0.5).to(td)
         B16 = ((torch.rand(N, K, generator=g) * 2 - 1) * K ** -0.5).to(td)
     else:
         A32 = torch.randn(M, K, generator=g)
-        if args.workload == "c3":  # 5 % outlier columns scaled x8
+        if workload == "c3":  # 5 % outlier columns scaled x8
             cols = torch.randperm(K, generator=g)[: (K * 5 + 99) // 100]
             A32[:, cols] *= 8
         A16 = A32.to(td)
@@ -172,12 +138,12 @@ def main():
         wall = (time.perf_counter() - t0) * 1e3 / steps
         return e0.elapsed_time(e1) / steps, wall
 
-    K_, W_ = args.steps, args.warmup
-    if args.steps_only:
+    K_, W_ = (max(5, args.steps // 2), max(3, args.warmup // 2)) if compact else (args.steps, args.warmup)
+    if args.steps_only and not compact:
         ms, _ = timed(step_overlapped, K_, W_)
         print(json.dumps({"steps_only": True, "steps": K_, "warmup": W_, "ms_per_step": ms}))
         return
-    if args.kernels_only:
+    if args.kernels_only and not compact:
         for fn in (gemm_alone, gemm_signal_alone, consumer_alone, norm):
             timed(fn, K_, W_)
             MM.zero_()
@@ -193,7 +159,7 @@ def main():
                 fn()
             torch.cuda.synchronize()
 
-    settle(step_serial)
+    settle(step_serial, 0.25 if compact else 0.5)
     ms_step, wall_step = timed(step_overlapped, K_, W_)
     ms_serial, _ = timed(step_serial, K_, W_)
     # second pass in the opposite order: what remains of drift between the two shows up here
@@ -211,10 +177,22 @@ def main():
     ACC.zero_()
     torch.cuda.synchronize()
 
+    flops = 2.0 * M * N * K
+    if compact:
+        gave_up = ov.status()
+        ov.close()
+        return {"workload": f"{workload}: {desc}", "dtype": dt, "cseg": cseg if len(cseg) <= 16 else f"{len(cseg)} x {cseg[0]}",
+                "gemm_alone_ms": ms_gemm, "gemm_signal_ms": ms_signal, "frac": flops / (ms_signal * 1e-3) / 1e12 / PEAK_TFLOPS,
+                "overlapped_ms": ms_step, "serial_ms": ms_serial,
+                "overlapped_vs_gemm_alone": ms_step / ms_gemm, "overlapped_vs_serial": ms_step / ms_serial,
+                "consumer_GBps": 6.0 * M * N / (ms_consumer * 1e-3) / 1e9,
+                "reorder_rmsnorm_GBps": (4.0 * bs * N + 2.0 * N) / (ms_norm * 1e-3) / 1e9,
+                "vendor_gemm_ms": ms_vendor, "waits_gave_up": gave_up}
+
     # wave-group-size sweep (large square only): group sizes in waves of 256 tiles;
     # 8 and 16 waves are a single group, i.e. the serial path (test/test.py:104)
     sweep = []
-    if args.workload == "c5" and not args.no_group_sweep:
+    if workload == "c5" and not args.no_group_sweep:
         for waves in (1, 2, 4, 8, 16):
             cs = fo.layout.cseg_from_waves(T, 256 * waves)
             if len(cs) == 1:
@@ -234,7 +212,7 @@ def main():
 
     # bf16 repeat of the large square: the same step with bf16 operands
     bf16_repeat = None
-    if args.workload == "c5" and dt == "f16" and not args.no_group_sweep:
+    if workload == "c5" and dt == "f16" and not args.no_group_sweep:
         tb = torch.bfloat16
         Ab, Bb, gb = A16.float().to(tb).cuda(), B16.float().to(tb).cuda(), gamma16.float().to(tb).cuda()
         Cb = torch.empty(M * N, device="cuda", dtype=tb)
@@ -266,7 +244,6 @@ def main():
         ov.set_accumulator(ACC)
         del Ab, Bb, Cb, Cbp, ACCb, Yb
 
-    flops = 2.0 * M * N * K
     achieved = flops / (ms_signal * 1e-3) / 1e12
     out = {
         "metric": "GEMM+signal+reorder TFLOP/s (% MFMA peak); overlapped vs serial time, 1 GPU",
@@ -276,7 +253,7 @@ def main():
         "ms_per_step": ms_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dt, "data": "synthetic",
-        "config": {"workload": f"{args.workload}: {desc}", "M": M, "N": N, "K": K, "tile": [BM, BN],
+        "config": {"workload": f"{workload}: {desc}", "M": M, "N": N, "K": K, "tile": [BM, BN],
                    "groups": len(cseg), "cseg": cseg if len(cseg) <= 16 else f"{len(cseg)} x {cseg[0]}", "algo": algo,
                    "consumer_launches": "on the GEMM stream behind the GEMM (automatic choice for a GEMM this short)"
                    if (args.fused < 0 and 2.0 * M * N * K < 6.4e10)
@@ -285,7 +262,11 @@ def main():
         "roofline": {"bound": "mfma", "kernel": "fo_gemm_kernel (signal epilogue)",
                      "achieved": achieved, "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_TFLOPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, dt))},
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((workload, dt)),
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE counter runs of this kernel and workload "
+                                       "(profiles/gemm_c5_hbm_traffic.md), not re-measured in this run; it moves by "
+                                       "about 10 % between runs"
+                     if (workload, dt) in MEASURED_TRAFFIC_BYTES else None},
         "times_ms": {"overlapped_step": ms_step, "overlapped_step_wall": wall_step,
                      "serial_step": ms_serial, "gemm_alone": ms_gemm, "gemm_signal_alone": ms_signal,
                      "consumer_alone": ms_consumer, "reorder_rmsnorm_alone": ms_norm,
@@ -301,6 +282,64 @@ def main():
         "bf16_repeat": bf16_repeat,
     }
 
+    out["waits_gave_up"] = ov.status()   # 1: a bounded device-side wait ran out of polls; the timings are then void
+    return out, ov, (A16, B16, gamma16, eps, M)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS))
+    ap.add_argument("--dtype", default=None, choices=["f16", "bf16"])
+    ap.add_argument("--swizzle", type=int, default=4)
+    ap.add_argument("--fused", type=int, default=-1,
+                    help="-1: library default (one wait+reduce launch above 16 groups), 0: two launches per "
+                         "group, 1: one launch")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--group-tiles", type=int, default=0, help="tiles per wave group (0: the workload's default)")
+    ap.add_argument("--no-group-sweep", action="store_true", help="skip the wave-group-size sweep (c5 only)")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="skip the compact records of the c2, c3 and c4 workloads that the default c5 run appends")
+    ap.add_argument("--kernels-only", action="store_true",
+                    help="run each hot kernel alone on one stream and exit: for counter collection, which "
+                         "serialises dispatches and would stall a waiter that spins on another queue")
+    ap.add_argument("--steps-only", action="store_true",
+                    help="enqueue warmup + steps overlapped steps and exit: for a kernel-trace timeline of the "
+                         "steady state")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run a 256 MiB device-to-device copy five times (reference point for "
+                         "scaling the FETCH_SIZE / WRITE_SIZE counters) and exit")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the collective is "
+              "replaced by a one-GPU consumer); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    os.environ.setdefault("FO_WAIT_MAX_POLLS", "200000000")  # a lost signal must not hang the GPU
+    import torch
+    import flashoverlap_amd as fo
+    from flashoverlap_amd import ops
+
+    torch.cuda.set_device(0)
+    if args.copy_calibration:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": src.numel(), "copy_bytes_written": dst.numel(), "copies": 5}))
+        return
+    res = measure(args, args.workload)
+    if res is None:  # --steps-only / --kernels-only printed their own line
+        return
+    out, ov, (A16, B16, gamma16, eps, M) = res
+    if args.workload == "c5" and not args.no_other_workloads:
+        ov.close()
+        ov = None
+        torch.cuda.empty_cache()
+        out["other_workloads"] = [measure(args, w, compact=True) for w in ("c2", "c3", "c4")]
     if not args.no_cpu_baseline:
         from oracle import cpu_baseline
         r = cpu_baseline.time_sample(A16, B16, gamma16, eps, target_seconds=15.0)
@@ -309,7 +348,10 @@ def main():
                                "sample": f"torch CPU fp32 matmul + RMSNorm on the first {r['rows']} of "
                                          f"{M} rows of the same A (all of B), {r['passes']} passes, {r['seconds']:.1f} s; "
                                          f"host has {os.cpu_count()} logical cpus"}
-    ov.close()
+    if ov is not None:
+        ov.close()
+    assert out["waits_gave_up"] == 0 and all(o["waits_gave_up"] == 0 for o in out.get("other_workloads", [])), \
+        "a device-side wait gave up: the step ran on incomplete tiles"
     print(json.dumps(out))
 
 

@@ -49,6 +49,9 @@ SIGNATURES = {
     "fo_overlap_set_world": (c_int, [vp, c_int, c_int]),
     "fo_overlap_set_accumulator": (c_int, [vp, vp, c_i64]),
     "fo_overlap_set_fused_consumer": (c_int, [vp, c_int]),
+    "fo_overlap_set_schedule": (c_int, [vp, ctypes.c_double, c_int]),
+    "fo_overlap_set_wait_limit": (c_int, [vp, c_i64]),
+    "fo_overlap_status": (c_int, [vp, vp]),
     "fo_overlap_comm_stream": (vp, [vp]),
     "fo_overlap_gemm": (c_int, [vp, c_int, c_int, c_int, c_int, vp, vp, vp, c_int]),
     "fo_overlap_gemm_allreduce": (c_int, [vp, c_int, c_int, c_int, c_int, vp, vp, vp, vp, vp, c_int,

@@ -63,18 +63,20 @@ int fo_pick_raster(int algo, int M, int N, fo_raster *r) {
     r->panel = e->f[10] < r->grid_m ? e->f[10] : r->grid_m;
     r->xcd_remap = (r->grid_m * r->grid_n >= 16) ? 1 : 0;
     r->tail_tiles = 0;
+    r->resident = 0;
     r->tail_sub_m = r->tail_sub_n = 1;
     if (r->mtm == 256 && r->mtn == 256) {
-        // The 256x256 launch is persistent on 256 workgroups (one per CU).  When at
-        // most half a wave is left after the last full one, those positions go to
-        // a second launch with the Algo's own tile, which fits them into a single
-        // wave of its own (512 resident workgroups of 128x128, 256 of 128x256 or
-        // 256x128).  Measured against one more wave of mostly idle CUs: +5 % on
+        // The 256x256 launch is persistent on as many workgroups as stay resident (one
+        // per CU: 256).  When at most half a wave is left after the last full one, those
+        // positions go to a second launch with the Algo's own tile, which fits them into a
+        // single wave of its own (two resident workgroups of 128x128 per CU, one of 128x256
+        // or 256x128).  Measured against one more wave of mostly idle CUs: +5 % on
         // 8192x7168x4096 (3.5 waves), +15 % on 4096x5120x4096 (1.25 waves).
-        const int resident = 256;
+        const int resident = fo_main_tile_resident();
+        r->resident = resident;
         const int nt = r->grid_m * r->grid_n, rem = nt % resident;
         const int per = (256 / bm) * (256 / bn);
-        if (nt > resident && rem != 0 && per > 1 && rem * per <= (per == 4 ? 512 : 256)) {
+        if (nt > resident && rem != 0 && per > 1 && rem * per <= (per == 4 ? 2 * resident : resident)) {
             r->tail_tiles = rem;
             r->tail_sub_m = 256 / bm;
             r->tail_sub_n = 256 / bn;
@@ -143,7 +145,7 @@ extern "C" const char *fo_error_string(int code) {
         case FO_ERR_ALGO: return "Algo index out of range";
         case FO_ERR_DTYPE: return "dtype must be FO_F16 or FO_BF16";
         case FO_ERR_SEGMENTS: return "cSeg does not partition the tiles (or too many groups for monitor mode)";
-        case FO_ERR_STATE: return "fo_overlap handle used before its init call";
+        case FO_ERR_STATE: return "fo_overlap handle used before its init call, or a launch that does not fit this device";
         default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
     }
 }

@@ -38,10 +38,12 @@ __global__ void fo_set_kernel(int32_t *word, int value) {
 // groups l, l + 256, ...  (a single lane walking 256 counters one after the
 // other measured 130 us on counters that were all complete already; one
 // wavefront with an acquiring CAS per group 4.5 us).  The resets are relaxed and
-// one acquire fence per lane follows them.
+// one acquire fence per lane follows them.  A lane whose bounded poll runs out
+// sets *status (if given) and leaves; its remaining groups keep their counts.
 constexpr int WAIT_GROUPS_THREADS = 256;
 __global__ __launch_bounds__(WAIT_GROUPS_THREADS) void fo_wait_groups_kernel(int count, const int32_t *expect,
-                                                                             int32_t *counters, long max_polls) {
+                                                                             int32_t *counters, long max_polls,
+                                                                             int32_t *status) {
     for (int g = threadIdx.x; g < count; g += blockDim.x) {
         const int want = expect[g];
         long polls = 0;
@@ -53,7 +55,10 @@ __global__ __launch_bounds__(WAIT_GROUPS_THREADS) void fo_wait_groups_kernel(int
                                                          __HIP_MEMORY_SCOPE_AGENT))
                     break;
             }
-            if (max_polls > 0 && ++polls >= max_polls) return;
+            if (max_polls > 0 && ++polls >= max_polls) {  // give up: flag it, leave the counter as it is
+                if (status) __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                return;
+            }
             __builtin_amdgcn_s_sleep(8);
         }
     }
@@ -465,12 +470,17 @@ int consumer_grid(long n16, bool stream_acc) {
 
 }  // namespace
 
-extern "C" int fo_wait(int expect, int32_t *counter, fo_stream_t stream) {
+// max_polls < 0: the bound from the environment (none when unset); 0: unbounded.
+int fo_wait_with(int expect, int32_t *counter, long max_polls, int32_t *status, fo_stream_t stream) {
     if (!counter) return FO_ERR_ARG;
     hipLaunchKernelGGL(fo_wait_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream), expect,
-                       counter, default_max_polls(), (int32_t *)nullptr);
+                       counter, max_polls < 0 ? default_max_polls() : max_polls, status);
     FO_LAUNCH_CHECK();
     return FO_OK;
+}
+
+extern "C" int fo_wait(int expect, int32_t *counter, fo_stream_t stream) {
+    return fo_wait_with(expect, counter, -1, nullptr, stream);
 }
 
 extern "C" int fo_set(int32_t *word, int value, fo_stream_t stream) {
@@ -480,19 +490,39 @@ extern "C" int fo_set(int32_t *word, int value, fo_stream_t stream) {
     return FO_OK;
 }
 
-extern "C" int fo_wait_groups(int count, const int32_t *expect_dev, int32_t *counters, fo_stream_t stream) {
+int fo_wait_groups_with(int count, const int32_t *expect_dev, int32_t *counters, long max_polls, int32_t *status,
+                        fo_stream_t stream) {
     if (count <= 0 || !expect_dev || !counters) return FO_ERR_ARG;
     hipLaunchKernelGGL(fo_wait_groups_kernel, dim3(1), dim3(count < WAIT_GROUPS_THREADS ? count : WAIT_GROUPS_THREADS), 0,
-                       static_cast<hipStream_t>(stream), count, expect_dev, counters, default_max_polls());
+                       static_cast<hipStream_t>(stream), count, expect_dev, counters,
+                       max_polls < 0 ? default_max_polls() : max_polls, status);
     FO_LAUNCH_CHECK();
     return FO_OK;
 }
 
+extern "C" int fo_wait_groups(int count, const int32_t *expect_dev, int32_t *counters, fo_stream_t stream) {
+    return fo_wait_groups_with(count, expect_dev, counters, -1, nullptr, stream);
+}
+
 extern "C" int fo_wait_bounded(int expect, int32_t *counter, int64_t max_polls, int32_t *status,
                                fo_stream_t stream) {
-    if (!counter || max_polls < 0) return FO_ERR_ARG;
-    hipLaunchKernelGGL(fo_wait_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream), expect,
-                       counter, (long)max_polls, status);
+    if (max_polls < 0) return FO_ERR_ARG;
+    return fo_wait_with(expect, counter, (long)max_polls, status, stream);
+}
+
+// Fills n words; the clearing step of callers that may be under stream capture,
+// where a memset node is avoided.
+namespace {
+__global__ void fo_fill_kernel(int32_t *words, int n, int value) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) words[i] = value;
+}
+}  // namespace
+
+int fo_fill_words(int32_t *words, int n, int value, fo_stream_t stream) {
+    if (!words || n <= 0) return FO_ERR_ARG;
+    const int blocks = (n + 255) / 256;
+    hipLaunchKernelGGL(fo_fill_kernel, dim3(blocks < 64 ? blocks : 64), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       words, n, value);
     FO_LAUNCH_CHECK();
     return FO_OK;
 }
@@ -584,7 +614,8 @@ extern "C" int fo_consumer_reduce(int dtype, const void *src, void *acc, int64_t
 int fo_wait_reduce_groups_with(int dtype, const void *C, void *ACC, int32_t *MM, const int32_t *cseg_dev, int G,
                                int64_t tile_elems, int W, int64_t seg_stride, void *own, int rank,
                                int32_t *workspace, int nblocks, int slices, int poll_gap_ns, bool stream_acc,
-                               fo_stream_t stream) {
+                               long max_polls, fo_stream_t stream) {
+    if (max_polls < 0) max_polls = default_max_polls();
     if (!MM || !cseg_dev || !workspace || G <= 0 || tile_elems <= 0 || W <= 0) return FO_ERR_ARG;
     if (ACC && !C) return FO_ERR_ARG;
     if (own && (!ACC || W < 2 || rank < 0 || rank >= W)) return FO_ERR_ARG;
@@ -604,12 +635,12 @@ int fo_wait_reduce_groups_with(int dtype, const void *C, void *ACC, int32_t *MM,
     if (dtype == FO_F16)
         hipLaunchKernelGGL(fo_wait_reduce_kernel<fo_f16_tag>, grid, block, 0, s, (const fo_u32x4 *)C,
                            (fo_u32x4 *)ACC, MM, cseg_dev, G, (long)(tile_elems / 8), W,
-                           (long)(seg_stride / 8), slices, workspace, default_max_polls(), sleep_ticks,
+                           (long)(seg_stride / 8), slices, workspace, max_polls, sleep_ticks,
                            (fo_u32x4 *)own, rank, (int)stream_acc);
     else if (dtype == FO_BF16)
         hipLaunchKernelGGL(fo_wait_reduce_kernel<fo_bf16_tag>, grid, block, 0, s, (const fo_u32x4 *)C,
                            (fo_u32x4 *)ACC, MM, cseg_dev, G, (long)(tile_elems / 8), W,
-                           (long)(seg_stride / 8), slices, workspace, default_max_polls(), sleep_ticks,
+                           (long)(seg_stride / 8), slices, workspace, max_polls, sleep_ticks,
                            (fo_u32x4 *)own, rank, (int)stream_acc);
     else
         return FO_ERR_DTYPE;
@@ -624,7 +655,7 @@ extern "C" int fo_wait_reduce_groups(int dtype, const void *C, void *ACC, int32_
                                      int64_t seg_stride, void *own, int rank, int32_t *workspace,
                                      int nblocks, int slices, int poll_gap_ns, fo_stream_t stream) {
     return fo_wait_reduce_groups_with(dtype, C, ACC, MM, cseg_dev, G, tile_elems, W, seg_stride, own, rank,
-                                      workspace, nblocks, slices, poll_gap_ns, false, stream);
+                                      workspace, nblocks, slices, poll_gap_ns, false, -1, stream);
 }
 
 extern "C" int fo_reorder_rmsnorm(int dtype, const void *X, void *Y, const void *Wt, int bs, int dim,

@@ -92,8 +92,11 @@ struct fo_raster {
     // second launch instead, with the Algo's own (smaller) tile: the last
     // tail_tiles positions of the raster, each cut into tail_sub_m x tail_sub_n.
     int tail_tiles, tail_sub_m, tail_sub_n;
+    int resident;  // workgroups of the 256x256 launch the tail split was computed for (0: not a 256x256 raster)
 };
 int fo_pick_raster(int algo, int M, int N, fo_raster *r);
+// Resident workgroups of the 256x256 kernel shape on the current device (fo_gemm.hip).
+int fo_main_tile_resident();
 
 // fo_gemm_signal / fo_gemm_scatter (RE != nullptr) without the counters: tiles are
 // stored reordered, MM is never touched (fo_gemm.hip; used by fo_overlap.cpp).
@@ -117,7 +120,17 @@ int fo_consumer_reduce_groups_with(int dtype, const void *src, void *acc, const 
 int fo_wait_reduce_groups_with(int dtype, const void *C, void *ACC, int32_t *MM, const int32_t *cseg_dev, int G,
                                int64_t tile_elems, int W, int64_t seg_stride, void *own, int rank,
                                int32_t *workspace, int nblocks, int slices, int poll_gap_ns, bool stream_acc,
-                               fo_stream_t stream);
+                               long max_polls, fo_stream_t stream);
+
+// The waits with their bound and status word chosen by the caller (fo_aux.hip).
+// max_polls < 0: the bound of the environment variable FO_WAIT_MAX_POLLS (none
+// when unset); 0: unbounded.  A wait that gives up stores 1 into *status (may be
+// null) and leaves its counter as it is.
+int fo_wait_with(int expect, int32_t *counter, long max_polls, int32_t *status, fo_stream_t stream);
+int fo_wait_groups_with(int count, const int32_t *expect_dev, int32_t *counters, long max_polls, int32_t *status,
+                        fo_stream_t stream);
+// words[0..n) = value by a small kernel (no memset node under stream capture).
+int fo_fill_words(int32_t *words, int n, int value, fo_stream_t stream);
 
 // Workgroup id -> macro tile coordinates; identical code on host and device.
 __host__ __device__ inline void fo_wg_to_tile(int wg, int grid_m, int grid_n, int panel,

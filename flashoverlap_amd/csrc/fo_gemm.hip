@@ -1,37 +1,55 @@
 // Host side of the gfx950 MFMA GEMM: picks the kernel shape for a problem and
 // launches it (plain, signal and scatter epilogues).  The device code is in
 // fo_gemm_kernel.h.
+#include <atomic>
+#include <mutex>
+
 #include "fo_gemm_kernel.h"
 
 namespace {
 
 using namespace fo_gemm_dev;
 
+constexpr int kMaxDevices = 64;
+
 // One compiled shape of the kernel template.  The launch is persistent: as many
 // workgroups as the device keeps resident at once (or fewer, if the problem has
 // fewer macro tiles); each walks the raster with that stride.
 // With `resident_out` set nothing is launched: the call only reports how many workgroups the
-// launch would hold, and in resident_out[1..3] the kernel's registers per lane, LDS bytes
-// and threads per workgroup.
+// launch would hold, in resident_out[1..3] the kernel's registers per lane, LDS bytes and
+// threads per workgroup, and in resident_out[4] how many workgroups stay resident at most.
+// expect_resident > 0: refuse (FO_ERR_STATE) unless that many stay resident.
 template <typename Tag, int MTM, int MTN, int BK, int SA, int SB, int WM, int WN, int MODE>
-int launch_variant(const GemmArgs &a, hipStream_t stream, int *resident_out) {
+int launch_variant(const GemmArgs &a, hipStream_t stream, int *resident_out, int expect_resident) {
     auto kern = fo_gemm_kernel<Tag, MTM, MTN, BK, SA, SB, WM, WN, MODE>;
     constexpr int smem = smem_bytes<MTM, MTN, BK, SA, SB>();
     constexpr int threads = WM * WN * 64;
-    static int resident = 0;  // per instantiation; the attribute is process wide
-    if (!resident) {
-        FO_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-        int dev = 0, cus = 0, per_cu = 0;
-        FO_HIP_CHECK(hipGetDevice(&dev));
-        FO_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-        FO_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(kern),
-                                                                  threads, smem));
-        if (cus <= 0 || per_cu <= 0) return FO_ERR_STATE;
-        // a multiple of 8 keeps "workgroup id mod 8 = XCD" true for every tile of the walk
-        resident = (cus * per_cu) / 8 * 8;
-        if (resident <= 0) resident = cus * per_cu;
+    // Resident workgroups of this instantiation per device; the LDS attribute is set once per device too.
+    static std::mutex mu;
+    static int resident_of[kMaxDevices];
+    int dev = 0;
+    FO_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return FO_ERR_STATE;
+    int resident;
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        if (!resident_of[dev]) {
+            FO_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+            int cus = 0, per_cu = 0;
+            FO_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+            FO_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(kern),
+                                                                      threads, smem));
+            if (cus <= 0 || per_cu <= 0) return FO_ERR_STATE;
+            // a multiple of 8 keeps "workgroup id mod 8 = XCD" true for every tile of the walk
+            int r = (cus * per_cu) / 8 * 8;
+            resident_of[dev] = r > 0 ? r : cus * per_cu;
+        }
+        resident = resident_of[dev];
     }
+    // The raster (and with it the schedule order handed to the caller as the hint) was laid out for
+    // expect_resident workgroups; a launch that would hold another number walks the tiles differently.
+    if (expect_resident > 0 && resident != expect_resident) return FO_ERR_STATE;
     const int ntiles = a.count;
     if (resident_out) {
         hipFuncAttributes attr;
@@ -40,6 +58,7 @@ int launch_variant(const GemmArgs &a, hipStream_t stream, int *resident_out) {
         resident_out[1] = attr.numRegs;
         resident_out[2] = smem;
         resident_out[3] = threads;
+        resident_out[4] = resident;
         return FO_OK;
     }
     dim3 grid(ntiles < resident ? ntiles : resident), block(threads);
@@ -48,26 +67,27 @@ int launch_variant(const GemmArgs &a, hipStream_t stream, int *resident_out) {
     return FO_OK;
 }
 
-// Macro tile -> kernel shape.  256x256 (eight wavefronts, three 32 KiB slots for
-// the A part and two for the B part of a K step: all 160 KiB) is the workhorse; the smaller shapes serve problems whose M or N is
-// not a multiple of 256 or that have too few 256x256 tiles to fill the chip.
+// Macro tile -> kernel shape.  256x256 (eight wavefronts, two 64 KiB slots of a K step's A and B
+// parts) is the workhorse; the smaller shapes (three slots for 128x256 and 256x128, two for 128x128)
+// serve problems whose M or N is not a multiple of 256 or that have too few 256x256 tiles to fill the chip.
 template <typename Tag, int MODE>
-int launch_tile(const GemmArgs &a, int mtm, int mtn, hipStream_t stream, int *resident_out) {
+int launch_tile(const GemmArgs &a, int mtm, int mtn, hipStream_t stream, int *resident_out, int expect_resident) {
     if (mtm == 256 && mtn == 256)
-        return launch_variant<Tag, 256, 256, 64, 2, 2, 2, 4, MODE>(a, stream, resident_out);
+        return launch_variant<Tag, 256, 256, 64, 2, 2, 2, 4, MODE>(a, stream, resident_out, expect_resident);
     if (mtm == 128 && mtn == 128)
-        return launch_variant<Tag, 128, 128, 64, 2, 2, 2, 2, MODE>(a, stream, resident_out);
+        return launch_variant<Tag, 128, 128, 64, 2, 2, 2, 2, MODE>(a, stream, resident_out, expect_resident);
     if (mtm == 128 && mtn == 256)
-        return launch_variant<Tag, 128, 256, 64, 3, 3, 2, 4, MODE>(a, stream, resident_out);
+        return launch_variant<Tag, 128, 256, 64, 3, 3, 2, 4, MODE>(a, stream, resident_out, expect_resident);
     if (mtm == 256 && mtn == 128)
-        return launch_variant<Tag, 256, 128, 64, 3, 3, 2, 2, MODE>(a, stream, resident_out);
+        return launch_variant<Tag, 256, 128, 64, 3, 3, 2, 2, MODE>(a, stream, resident_out, expect_resident);
     return FO_ERR_ALGO;
 }
 
 template <int MODE>
-int launch_dtype(int dtype, const GemmArgs &a, int mtm, int mtn, hipStream_t stream, int *resident_out = nullptr) {
-    if (dtype == FO_F16) return launch_tile<fo_f16_tag, MODE>(a, mtm, mtn, stream, resident_out);
-    if (dtype == FO_BF16) return launch_tile<fo_bf16_tag, MODE>(a, mtm, mtn, stream, resident_out);
+int launch_dtype(int dtype, const GemmArgs &a, int mtm, int mtn, hipStream_t stream, int *resident_out = nullptr,
+                 int expect_resident = 0) {
+    if (dtype == FO_F16) return launch_tile<fo_f16_tag, MODE>(a, mtm, mtn, stream, resident_out, expect_resident);
+    if (dtype == FO_BF16) return launch_tile<fo_bf16_tag, MODE>(a, mtm, mtn, stream, resident_out, expect_resident);
     return FO_ERR_DTYPE;
 }
 
@@ -107,24 +127,52 @@ int run_gemm(int mode, int dtype, int M, int N, int K, int rLDN, const int32_t *
         if (monitor && G > a.TN - 1) return FO_ERR_SEGMENTS;
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    auto launch = [&](const GemmArgs &g, int mtm, int mtn) {
+    auto launch = [&](const GemmArgs &g, int mtm, int mtn, int expect) {
         switch (mode) {
-            case MODE_PLAIN: return launch_dtype<MODE_PLAIN>(dtype, g, mtm, mtn, s);
-            case MODE_SIGNAL: return launch_dtype<MODE_SIGNAL>(dtype, g, mtm, mtn, s);
-            default: return launch_dtype<MODE_SCATTER>(dtype, g, mtm, mtn, s);
+            case MODE_PLAIN: return launch_dtype<MODE_PLAIN>(dtype, g, mtm, mtn, s, nullptr, expect);
+            case MODE_SIGNAL: return launch_dtype<MODE_SIGNAL>(dtype, g, mtm, mtn, s, nullptr, expect);
+            default: return launch_dtype<MODE_SCATTER>(dtype, g, mtm, mtn, s, nullptr, expect);
         }
     };
-    rc = launch(a, r.mtm, r.mtn);
+    // the tail split was computed for r.resident workgroups of the main launch
+    rc = launch(a, r.mtm, r.mtn, r.tail_tiles ? r.resident : 0);
     if (rc || !r.tail_tiles) return rc;
     // the last, partial wave of 256x256 tiles: the same raster positions in the Algo's own tile
     GemmArgs t = a;
     t.first = a.count;
     t.sub_m = r.tail_sub_m; t.sub_n = r.tail_sub_n;
     t.count = r.tail_tiles * r.tail_sub_m * r.tail_sub_n;
-    return launch(t, a.BM, a.BN);
+    return launch(t, a.BM, a.BN, 0);
 }
 
 }  // namespace
+
+// Workgroups of the 256x256 shape that stay resident on the current device: what the
+// raster's tail split is computed from.  All epilogues and both dtypes of that shape use
+// the same LDS (one workgroup per CU); the launch checks its own instantiation against
+// this number.  Without a usable device (host-only callers asking for the schedule order)
+// the answer is MI355X's: 256 CUs, one workgroup each.
+int fo_main_tile_resident() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    static std::atomic<int> cached[kMaxDevices];  // asked on every launch: answered from here after the first
+    if (dev >= 0 && dev < kMaxDevices) {
+        const int c = cached[dev].load(std::memory_order_relaxed);
+        if (c > 0) return c;
+    }
+    GemmArgs a = {};
+    a.count = 1 << 30;
+    int info[5] = {0, 0, 0, 0, 0};
+    if (launch_dtype<MODE_SIGNAL>(FO_F16, a, 256, 256, nullptr, info) != FO_OK || info[4] <= 0) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    if (dev >= 0 && dev < kMaxDevices) cached[dev].store(info[4], std::memory_order_relaxed);
+    return info[4];
+}
 
 // The reordered (optionally row-mapped) store of the signalling GEMMs without
 // their counters, for a caller that orders GEMM and consumer by the stream alone.
@@ -146,7 +194,7 @@ extern "C" int fo_gemm_wave_tiles(int dtype, int algo, int M, int N, int32_t *ti
     a.grid_m = r.grid_m;
     a.grid_n = r.grid_n;
     a.count = r.grid_m * r.grid_n - r.tail_tiles;
-    int info[4] = {0, 0, 0, 0};
+    int info[5] = {0, 0, 0, 0, 0};
     rc = launch_dtype<MODE_SIGNAL>(dtype, a, r.mtm, r.mtn, nullptr, info);
     if (rc) return rc;
     *tiles = info[0] * (r.mtm / e->f[0]) * (r.mtn / e->f[1]);
@@ -162,7 +210,7 @@ extern "C" int fo_gemm_kernel_info(int dtype, int algo, int M, int N, int epilog
     a.grid_m = r.grid_m;
     a.grid_n = r.grid_n;
     a.count = r.grid_m * r.grid_n - r.tail_tiles;
-    int out[4] = {0, 0, 0, 0};
+    int out[5] = {0, 0, 0, 0, 0};
     switch (epilogue) {
         case MODE_PLAIN: rc = launch_dtype<MODE_PLAIN>(dtype, a, r.mtm, r.mtn, nullptr, out); break;
         case MODE_SIGNAL: rc = launch_dtype<MODE_SIGNAL>(dtype, a, r.mtm, r.mtn, nullptr, out); break;

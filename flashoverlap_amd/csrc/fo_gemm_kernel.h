@@ -101,8 +101,8 @@ __device__ __forceinline__ void wait_vmcnt() {
 // count, which can only make its waits longer, never shorter).  The
 // write-through form (system-scope cache policy) is used for the signalled
 // epilogues: the tile must be visible to other XCDs before its counter is
-// bumped, and a tile that never becomes dirty in L2 makes the releasing
-// write-back that precedes the signal nearly free.  The trailing s_nop covers
+// bumped, and a tile that never becomes dirty in L2 needs no releasing
+// write-back before the signal.  The trailing s_nop covers
 // the wait states gfx9 requires between a VMEM store of more than 8 bytes and a
 // VALU write of its data registers.
 __device__ __forceinline__ void store16_write_through(void *ptr, fo_u32x4 v) {
@@ -155,7 +155,10 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
     // LDS: stage-major, A part then B part; with SA = SB + 1 the last stage has an A part only
     constexpr int RING16 = SB * STAGE16 + (SA - SB) * A16;
     // vector memory instructions that may stay in flight when the next K step's operands are needed:
-    // everything requested after that step's last part (request order per step: B part, then A part)
+    // everything requested after that step's last part (request order per step: B part, then A part).
+    // Waiting with a non-zero count relies on vmcnt retiring this wavefront's loads and stores in
+    // issue order, as it does on gfx9-family parts (one counter for both, decremented in order): when
+    // vmcnt(n) returns, everything but the youngest n instructions has completed.
     constexpr int ALLOW = (SA - SB) * PA + (SB - 2) * P;
     constexpr int KK = BK / 32;                                  // MFMA k-steps per stage
     // epilogue: per-wavefront strip of 32 rows x WTN columns in the ring behind slot 0
@@ -695,9 +698,10 @@ __global__ __launch_bounds__(WM *WN * 64) void fo_gemm_kernel(GemmArgs p) {
                     prev_gs[s] = gs[s];
                 }
             } else {
-                // Every lane waits until its own stores are acknowledged, the
-                // barrier collects the workgroup, and only then one lane
-                // releases at agent scope and bumps the group counter.  The
+                // Every lane waits until its own write-through stores are
+                // acknowledged, the barrier collects the workgroup, and only then
+                // one lane bumps the group counter (a relaxed atomic: the tile is
+                // in memory already, there is nothing left to release).  The
                 // reference has no fence here (src/overlap/gemm_with_signal.h:337-351).
                 __builtin_amdgcn_s_waitcnt(0);
                 __builtin_amdgcn_s_barrier();

@@ -1,55 +1,82 @@
 // Host orchestration of the overlap path: the counterpart of class OverlapImpl
 // (src/overlap_impl.h:12-43, src/overlap_impl.cu) behind a C handle.  Two HIP
 // streams; every call only enqueues work and returns.  May be captured into a HIP graph.
+#include <mutex>
 #include <new>
 
 #include "fo_common.h"
 
-struct fo_overlap {
-    hipStream_t gemm_stream = nullptr;
-    hipStream_t comm_stream = nullptr;
-    hipEvent_t forked = nullptr, joined = nullptr;  // used only while the GEMM stream is being captured
-    int32_t *workspace = nullptr;  // zeroed words of the one-launch wait+reduce kernel
-    bool gemm_ready = false;
-    bool overlap_ready = false;
-    int rank = 0, world = 1;
-    void *acc = nullptr;
-    int64_t acc_nelem = 0;
-    int fused = -1;  // -1: choose per call (one launch when there are many groups)
-};
-
 namespace {
 
-// Two launches per group cost a few microseconds each; beyond this many groups
-// the single wait+reduce launch is the faster consumer.  With few, large groups
-// the per-group launches win: a kernel that starts when its group is complete
-// needs no polling workgroups resident beside the GEMM.
-constexpr int kFusedFromGroups = 16;
+// Words of the workspace (device int32[kWorkspaceWords], zero between calls).
+enum {
+    kWsLeft = 0,    // workgroups of the one-launch consumer that have left
+    kWsGaveUp = 1,  // set by any bounded wait of a call that ran out of polls
+    kWsJoin = 4,    // consumer stream -> GEMM stream
+    kWsFork = 5,    // GEMM stream -> consumer stream
+    kWorkspaceWords = 16,
+};
 
-// In automatic mode a GEMM shorter than this many flop (about 50 us of this
+// Defaults of the scheduling choices below; a handle can override them
+// (fo_overlap_set_schedule), they are measurements on one MI355X, not laws.
+//
+// Two launches per group cost a few microseconds each; beyond kFusedFromGroups
+// groups the single wait+reduce launch is the faster consumer.  With few, large
+// groups the per-group launches win: a kernel that starts when its group is
+// complete needs no polling workgroups resident beside the GEMM.
+//
+// In automatic mode a GEMM shorter than kInStreamBelowFlop (about 50 us of this
 // GPU) keeps the whole call on the GEMM stream: the GEMM with its reordered
 // store and one consumer launch (with the monitor on: the signalling GEMM and
 // one wait that resets every counter between them).  Fork, join and pollers beside the
 // GEMM cost more than such a GEMM can hide (4096x4096x512 with 256 groups:
 // 71 us overlapped, 48 us in stream).
+//
+// kGemmFlopPerNs: what a GEMM is expected to sustain, for sizing the pause
+// between polls only.
+constexpr int kFusedFromGroups = 16;
 constexpr double kInStreamBelowFlop = 6.4e10;
+constexpr double kGemmFlopPerNs = 1.2e6;
+
+}  // namespace
+
+struct fo_overlap {
+    hipStream_t gemm_stream = nullptr;
+    hipStream_t comm_stream = nullptr;  // null: every call stays on the GEMM stream
+    hipEvent_t forked = nullptr, joined = nullptr;  // used only while the GEMM stream is being captured
+    int32_t *workspace = nullptr;
+    bool gemm_ready = false;
+    bool overlap_ready = false;
+    int rank = 0, world = 1;
+    void *acc = nullptr;
+    int64_t acc_nelem = 0;
+    int fused = -1;        // -1: choose per call (one launch when there are many groups)
+    long max_polls = -1;   // bound of every device-side wait; -1: FO_WAIT_MAX_POLLS, 0: none
+    int fused_from_groups = kFusedFromGroups;
+    double in_stream_below_flop = kInStreamBelowFlop;
+    int token = 1;         // value the fork and join words carry from one stream to the other
+    bool always_fork = false;  // the consumer stream must not start before this call's first kernel on the GEMM stream
+};
+
+namespace {
 
 bool in_stream(const fo_overlap *h, int M, int N, int K) {
-    return h->fused < 0 && 2.0 * M * N * K < kInStreamBelowFlop;
+    if (!h->comm_stream) return true;
+    return h->fused < 0 && 2.0 * M * N * K < h->in_stream_below_flop;
 }
 
 int fused_grid(const fo_overlap *h, int G) {  // 0: per-group launches, otherwise workgroups of the one launch
-    if (h->fused < 0) return G > kFusedFromGroups ? 256 : 0;
+    if (h->fused < 0) return G > h->fused_from_groups ? 256 : 0;
     if (h->fused == 1) return 256;
     return h->fused;
 }
 
 // Pause between a workgroup's polls in the one-launch consumer: 100 ns per
 // workgroup keeps the GEMM's slowdown near one percent, but no more than about
-// a sixtieth of the GEMM's expected duration (at 1.2 PFLOP/s), so that a short
-// problem is not left waiting for a sleeping poller.
+// a sixtieth of the GEMM's expected duration, so that a short problem is not
+// left waiting for a sleeping poller.
 int fused_poll_gap_ns(int M, int N, int K, int grid) {
-    const double gemm_ns = 2.0 * M * N * K / 1.2e6;
+    const double gemm_ns = 2.0 * M * N * K / kGemmFlopPerNs;
     double gap = grid * 100.0;
     if (gap > gemm_ns / 60) gap = gemm_ns / 60;
     if (gap < 500) gap = 500;
@@ -107,20 +134,21 @@ bool capturing(const fo_overlap *h) {
 // reference's wait kernels may start early: a single sleeping lane disturbs nobody).
 int fork(fo_overlap *h, bool captured, bool polling_consumer) {
     if (captured) {
+        if (!h->forked || !h->joined) return FO_ERR_STATE;  // a handle-free call has no events to capture with
         FO_HIP_CHECK(hipEventRecord(h->forked, h->gemm_stream));
         FO_HIP_CHECK(hipStreamWaitEvent(h->comm_stream, h->forked, 0));
         return FO_OK;
     }
-    if (!polling_consumer) return FO_OK;
-    int rc = fo_set(h->workspace + 5, 1, h->gemm_stream);
+    if (!polling_consumer && !h->always_fork) return FO_OK;
+    int rc = fo_set(h->workspace + kWsFork, h->token, h->gemm_stream);
     if (rc) return rc;
-    return fo_wait(1, h->workspace + 5, h->comm_stream);
+    return fo_wait_with(h->token, h->workspace + kWsFork, h->max_polls, h->workspace + kWsGaveUp, h->comm_stream);
 }
 
 // consumer stream -> GEMM stream.  The reference records an event on the consumer stream
 // and makes the GEMM stream wait for it (src/overlap_impl.cu:260-263); an event wait across
 // queues measured about 12 us here, so outside a capture the join goes through memory: a
-// one-lane kernel at the end of the consumer stream sets workspace word 4 (stream order
+// one-lane kernel at the end of the consumer stream sets the workspace's join word (stream order
 // makes all earlier work there complete and visible first), a one-lane wait behind the
 // GEMM on the GEMM's stream consumes it.  The wait cannot start before the GEMM has ended
 // and everything it waits for was enqueued before it; the GEMM stream continues about 4 us
@@ -131,9 +159,9 @@ int join(fo_overlap *h, bool captured) {
         FO_HIP_CHECK(hipStreamWaitEvent(h->gemm_stream, h->joined, 0));
         return FO_OK;
     }
-    int rc = fo_set(h->workspace + 4, 1, h->comm_stream);
+    int rc = fo_set(h->workspace + kWsJoin, h->token, h->comm_stream);
     if (rc) return rc;
-    return fo_wait(1, h->workspace + 4, h->gemm_stream);
+    return fo_wait_with(h->token, h->workspace + kWsJoin, h->max_polls, h->workspace + kWsGaveUp, h->gemm_stream);
 }
 
 }  // namespace
@@ -193,8 +221,8 @@ extern "C" int fo_overlap_init(fo_overlap_t *h) {
     FO_HIP_CHECK(hipStreamCreateWithFlags(&h->comm_stream, hipStreamNonBlocking));
     FO_HIP_CHECK(hipEventCreateWithFlags(&h->forked, hipEventDisableTiming));
     FO_HIP_CHECK(hipEventCreateWithFlags(&h->joined, hipEventDisableTiming));
-    FO_HIP_CHECK(hipMalloc(&h->workspace, 64));
-    FO_HIP_CHECK(hipMemset(h->workspace, 0, 64));
+    FO_HIP_CHECK(hipMalloc(&h->workspace, kWorkspaceWords * sizeof(int32_t)));
+    FO_HIP_CHECK(hipMemset(h->workspace, 0, kWorkspaceWords * sizeof(int32_t)));
     h->overlap_ready = true;
     return FO_OK;
 }
@@ -219,6 +247,31 @@ extern "C" int fo_overlap_set_fused_consumer(fo_overlap_t *h, int fused) {
     return FO_OK;
 }
 
+extern "C" int fo_overlap_set_wait_limit(fo_overlap_t *h, int64_t max_polls) {
+    if (!h || max_polls < -1) return FO_ERR_ARG;
+    h->max_polls = (long)max_polls;
+    return FO_OK;
+}
+
+extern "C" int fo_overlap_set_schedule(fo_overlap_t *h, double in_stream_below_flop, int fused_from_groups) {
+    if (!h) return FO_ERR_ARG;
+    h->in_stream_below_flop = in_stream_below_flop < 0 ? kInStreamBelowFlop : in_stream_below_flop;
+    h->fused_from_groups = fused_from_groups < 0 ? kFusedFromGroups : fused_from_groups;
+    return FO_OK;
+}
+
+extern "C" int fo_overlap_status(fo_overlap_t *h, int32_t *gave_up) {
+    if (!h || !gave_up) return FO_ERR_ARG;
+    *gave_up = 0;
+    if (!h->overlap_ready) return FO_OK;
+    FO_HIP_CHECK(hipStreamSynchronize(h->comm_stream));
+    if (h->gemm_ready) FO_HIP_CHECK(hipStreamSynchronize(h->gemm_stream));
+    FO_HIP_CHECK(hipMemcpy(gave_up, h->workspace + kWsGaveUp, sizeof(int32_t), hipMemcpyDeviceToHost));
+    // A wait that gave up may have left the fork or join word set; both streams are idle now.
+    if (*gave_up) FO_HIP_CHECK(hipMemset(h->workspace, 0, kWorkspaceWords * sizeof(int32_t)));
+    return FO_OK;
+}
+
 extern "C" fo_stream_t fo_overlap_comm_stream(fo_overlap_t *h) {
     return h ? static_cast<fo_stream_t>(h->comm_stream) : nullptr;
 }
@@ -230,13 +283,13 @@ extern "C" int fo_overlap_gemm(fo_overlap_t *h, int dtype, int M, int N, int K, 
     return fo_gemm(dtype, M, N, K, A, B, C, algo, h->gemm_stream);
 }
 
-extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int N, int K,
-                                         const void *A, const void *B, void *C, int32_t *MM,
-                                         const int32_t *RA, int TM, int TN, int rLDN,
-                                         const int32_t *cseg_host, const int32_t *cseg_dev, int G,
-                                         int algo, int monitor) {
-    if (!h || !MM) return FO_ERR_ARG;
-    if (!h->gemm_ready || !h->overlap_ready) return FO_ERR_STATE;
+namespace {
+
+// GemmAllReduceOverlap on whatever `h` describes: a caller's handle, or the
+// streams and static workspace of a handle-free call.
+int allreduce_overlap(fo_overlap *h, int dtype, int M, int N, int K, const void *A, const void *B, void *C,
+                      int32_t *MM, const int32_t *RA, int TM, int TN, int rLDN, const int32_t *cseg_host,
+                      const int32_t *cseg_dev, int G, int algo, int monitor) {
     int32_t info[12];
     int rc = fo_algo_info(algo, info);
     if (rc) return rc;
@@ -270,14 +323,14 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
                                          h->gemm_stream)
                : fo_gemm_signal(dtype, M, N, K, rLDN, cseg_dev, G, A, B, C, MM, RA, monitor, algo,
                                 h->gemm_stream);
-    if (rc) return rc;  // nothing has been enqueued on the consumer stream yet
+    if (rc) return rc;  // the GEMM was refused: nothing of this call follows on either stream
 
     // C' and the accumulator together against the memory-side cache
     const bool stream_acc = fo_streams((int64_t)M * N * 4);
     if (fused) {
         rc = fo_wait_reduce_groups_with(dtype, C, h->acc, MM, cseg_dev, G, tile_elems, 1, 0, nullptr, 0,
                                         h->workspace, fused, fused_slices((int64_t)M * N, G, fused),
-                                        fused_poll_gap_ns(M, N, K, fused), stream_acc, h->comm_stream);
+                                        fused_poll_gap_ns(M, N, K, fused), stream_acc, h->max_polls, h->comm_stream);
         if (rc) return rc;
     } else {
         int64_t off = 0;
@@ -290,8 +343,9 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
             for (int g = i; g < j; g++) tiles += cseg_host[g];
             const int64_t n = tiles * tile_elems;
             if (!quiet) {
-                rc = j - i == 1 ? fo_wait(cseg_host[i], MM + i, cstream)  // resets the counter
-                                : fo_wait_groups(j - i, cseg_dev + i, MM + i, cstream);
+                int32_t *gave_up = h->workspace ? h->workspace + kWsGaveUp : nullptr;
+                rc = j - i == 1 ? fo_wait_with(cseg_host[i], MM + i, h->max_polls, gave_up, cstream)  // resets the counter
+                                : fo_wait_groups_with(j - i, cseg_dev + i, MM + i, h->max_polls, gave_up, cstream);
                 if (rc) return rc;
             }
             if (acc) {  // the groups of a batch are one contiguous range
@@ -304,6 +358,19 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
         }
     }
     return same_stream ? FO_OK : join(h, captured);
+}
+
+}  // namespace
+
+extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int N, int K,
+                                         const void *A, const void *B, void *C, int32_t *MM,
+                                         const int32_t *RA, int TM, int TN, int rLDN,
+                                         const int32_t *cseg_host, const int32_t *cseg_dev, int G,
+                                         int algo, int monitor) {
+    if (!h || !MM) return FO_ERR_ARG;
+    if (!h->gemm_ready || !h->overlap_ready) return FO_ERR_STATE;
+    return allreduce_overlap(h, dtype, M, N, K, A, B, C, MM, RA, TM, TN, rLDN, cseg_host, cseg_dev, G, algo,
+                             monitor);
 }
 
 extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, int N, int K,
@@ -360,7 +427,7 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
         rc = fo_wait_reduce_groups_with(dtype, C, h->acc, MM, cseg_dev, G, tile_elems, W, seg_stride,
                                         own_in_consumer ? D : nullptr, h->rank, h->workspace, fused,
                                         fused_slices((int64_t)M * N, G, fused), fused_poll_gap_ns(M, N, K, fused),
-                                        stream_acc, cstream);
+                                        stream_acc, h->max_polls, cstream);
         if (rc) return rc;
     }
     int64_t off = 0;
@@ -368,8 +435,9 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
     for (int i = 0; i < G;) {
         const int j = fused ? i + 1 : batch_end(cseg_host, G, i, done, wave);
         if (!fused && !quiet) {
-            rc = j - i == 1 ? fo_wait(cseg_host[i], MM + i, cstream)
-                            : fo_wait_groups(j - i, cseg_dev + i, MM + i, cstream);
+            int32_t *gave_up = h->workspace ? h->workspace + kWsGaveUp : nullptr;
+            rc = j - i == 1 ? fo_wait_with(cseg_host[i], MM + i, h->max_polls, gave_up, cstream)
+                            : fo_wait_groups_with(j - i, cseg_dev + i, MM + i, h->max_polls, gave_up, cstream);
             if (rc) return rc;
         }
         if (!fused && acc && W > 1 && j - i > 1) {

@@ -12,6 +12,7 @@
 #include <torch/custom_class.h>
 #include <torch/library.h>
 
+#include <algorithm>
 #include <vector>
 
 #include "flashoverlap.h"
@@ -60,11 +61,40 @@ Shape gemm_shape(const at::Tensor &A, const at::Tensor &B, const at::Tensor &C) 
     return {(int)A.size(0), (int)B.size(0), (int)A.size(1)};
 }
 
+// The kernels index MM, RA, RE and D through raw pointers; the reference checks none of
+// their sizes and overruns MM when there are more groups than tile columns
+// (test/test.py:94 allocates TN ints).  Refuse before anything is launched.
+void check_buffers(const Shape &s, int64_t Algo, const at::Tensor &MM, const at::Tensor &RA, int64_t rLDN,
+                   const at::Tensor &cSEG_CPU, const at::Tensor &cSEG_GPU, bool monitor, const at::Tensor *RE,
+                   const at::Tensor *D, int64_t world) {
+    int32_t info[12];
+    check(fo_algo_info((int)Algo, info), "Algo lookup");
+    TORCH_CHECK(s.M % info[0] == 0 && s.N % info[1] == 0, "flashoverlap: M x N = ", s.M, " x ", s.N,
+                " is not a multiple of the Algo's tile ", info[0], " x ", info[1]);
+    const int64_t TM = s.M / info[0], TN = s.N / info[1], G = cSEG_GPU.numel();
+    TORCH_CHECK(RA.dim() == 2 && RA.size(0) == TM && RA.size(1) == TN, "flashoverlap: RA must be [", TM, ", ", TN,
+                "] for this Algo");
+    TORCH_CHECK(cSEG_CPU.numel() == G, "flashoverlap: cSEG_CPU/cSEG_GPU differ");
+    const int64_t need = monitor ? (TM + 1) * TN : std::max(G, TN);
+    TORCH_CHECK(MM.numel() >= need, "flashoverlap: MM holds ", MM.numel(), " counters, ", need, " are needed (", G,
+                " groups, ", TM, " x ", TN, " tiles", monitor ? ", monitor)" : ")");
+    TORCH_CHECK(rLDN > 0 && (TM * TN) % rLDN == 0, "flashoverlap: rLDN = ", rLDN, " does not divide the tiles");
+    if (RE) {
+        const int64_t rows = (int64_t)s.M * s.N / (rLDN * info[1]);
+        TORCH_CHECK(RE->numel() >= rows, "flashoverlap: RE holds ", RE->numel(), " rows, the reshaped output has ",
+                    rows);
+    }
+    if (D) {
+        TORCH_CHECK(world > 0 && D->numel() >= (int64_t)s.M * s.N / world, "flashoverlap: D holds ", D->numel(),
+                    " elements, M*N/W = ", (int64_t)s.M * s.N / world, " are needed");
+    }
+}
+
 // class OverlapImpl, src/overlap_impl.h:12-43.
 struct OverlapImpl : torch::CustomClassHolder {
     fo_overlap_t *h = nullptr;
     at::Tensor acc;  // keeps the accumulation buffer alive
-    int64_t rank_ = 0;
+    int64_t rank_ = 0, world_ = 1;
 
     OverlapImpl() { check(fo_overlap_create(&h), "fo_overlap_create"); }
     ~OverlapImpl() override { fo_overlap_destroy(h); }
@@ -72,6 +102,7 @@ struct OverlapImpl : torch::CustomClassHolder {
     void nccl_init(int64_t rank, int64_t world, std::vector<int64_t> /*id*/) {
         check(fo_overlap_set_world(h, (int)rank, (int)world), "nccl_init");
         rank_ = rank;
+        world_ = world;
     }
     void cutlass_init() { check(fo_overlap_set_gemm_stream(h, current_stream()), "cutlass_init"); }
     void overlap_init() { check(fo_overlap_init(h), "overlap_init"); }
@@ -87,8 +118,8 @@ struct OverlapImpl : torch::CustomClassHolder {
                                 int64_t rLDN, at::Tensor cSEG_CPU, at::Tensor cSEG_GPU, int64_t Algo,
                                 bool if_monitor) {
         Shape s = gemm_shape(A, B, C);
-        TORCH_CHECK(RA.dim() == 2, "flashoverlap: RA must be [TM, TN]");
-        TORCH_CHECK(cSEG_CPU.numel() == cSEG_GPU.numel(), "flashoverlap: cSEG_CPU/cSEG_GPU differ");
+        check_buffers(s, Algo, MM, RA, rLDN, cSEG_CPU, cSEG_GPU, if_monitor, nullptr, nullptr, 1);
+        TORCH_CHECK(!acc.defined() || acc.numel() >= (int64_t)s.M * s.N, "flashoverlap: the accumulator is smaller than M*N");
         check(fo_overlap_gemm_allreduce(h, dtype_of(A), s.M, s.N, s.K, dev_ptr(A, "A"), dev_ptr(B, "B"),
                                         dev_ptr(C, "C"), dev_i32(MM, "MM"), dev_i32(RA, "RA"),
                                         (int)RA.size(0), (int)RA.size(1), (int)rLDN,
@@ -102,9 +133,9 @@ struct OverlapImpl : torch::CustomClassHolder {
                                     at::Tensor cSEG_CPU, at::Tensor cSEG_GPU, int64_t Algo,
                                     bool if_monitor) {
         Shape s = gemm_shape(A, B, C);
-        TORCH_CHECK(RA.dim() == 2, "flashoverlap: RA must be [TM, TN]");
-        TORCH_CHECK(cSEG_CPU.numel() == cSEG_GPU.numel(), "flashoverlap: cSEG_CPU/cSEG_GPU differ");
         TORCH_CHECK(D.scalar_type() == C.scalar_type(), "flashoverlap: C and D must share one dtype");
+        check_buffers(s, Algo, MM, RA, rLDN, cSEG_CPU, cSEG_GPU, if_monitor, &RE, &D, world_);
+        TORCH_CHECK(!acc.defined() || acc.numel() >= (int64_t)s.M * s.N, "flashoverlap: the accumulator is smaller than M*N");
         check(fo_overlap_gemm_reducescatter(
                   h, dtype_of(A), s.M, s.N, s.K, dev_ptr(A, "A"), dev_ptr(B, "B"), dev_ptr(C, "C"),
                   dev_ptr(D, "D"), dev_i32(MM, "MM"), dev_i32(RA, "RA"), dev_i32(RE, "RE"),
@@ -135,6 +166,8 @@ struct OverlapImpl : torch::CustomClassHolder {
     // NcclAllReduce, src/overlap_impl.cu:143-151.
     void nccl_allreduce(at::Tensor C) {
         if (!acc.defined()) return;  // a one-rank sum is the identity
+        TORCH_CHECK(acc.numel() >= C.numel() && acc.scalar_type() == C.scalar_type(),
+                    "flashoverlap: the accumulator must hold C.numel() elements of C's dtype");
         check(fo_consumer_reduce(dtype_of(C), dev_ptr(C, "C"), acc.data_ptr(), C.numel(),
                                  current_stream()),
               "nccl_allreduce");
@@ -159,9 +192,16 @@ struct OverlapImpl : torch::CustomClassHolder {
         acc = at::Tensor();
         check(fo_overlap_set_accumulator(h, nullptr, 0), "clear_accumulator");
     }
-    // addition: one wait+reduce launch for all groups instead of two launches per group.
-    void set_fused_consumer(bool fused) {
-        check(fo_overlap_set_fused_consumer(h, fused ? 1 : 0), "set_fused_consumer");
+    // addition: -1 chosen per call (default), 0 two launches per group as the reference's host loop,
+    // 1 one wait+reduce launch for all groups, n > 1 the same with n workgroups.
+    void set_fused_consumer(int64_t fused) {
+        check(fo_overlap_set_fused_consumer(h, (int)fused), "set_fused_consumer");
+    }
+    // addition: whether a bounded device-side wait gave up since the last query (synchronises).
+    int64_t status() {
+        int32_t gave_up = 0;
+        check(fo_overlap_status(h, &gave_up), "status");
+        return gave_up;
     }
 
    private:
@@ -200,6 +240,8 @@ struct BaselineImpl : torch::CustomClassHolder {
     }
     void nccl_allreduce(at::Tensor C) {
         if (!acc.defined()) return;
+        TORCH_CHECK(acc.numel() >= C.numel() && acc.scalar_type() == C.scalar_type(),
+                    "flashoverlap: the accumulator must hold C.numel() elements of C's dtype");
         check(fo_consumer_reduce(dtype_of(C), dev_ptr(C, "C"), acc.data_ptr(), C.numel(),
                                  current_stream()),
               "nccl_allreduce");
@@ -222,6 +264,11 @@ void reorder_rmsnorm_eps(at::Tensor X, at::Tensor RX, at::Tensor RW, int64_t BM,
     TORCH_CHECK(X.dim() == 2 && RX.sizes() == X.sizes(), "flashoverlap: X and RX must be [bs, dim]");
     TORCH_CHECK(X.scalar_type() == RX.scalar_type() && X.scalar_type() == RW.scalar_type(),
                 "flashoverlap: X, RX and RW must share one dtype");
+    TORCH_CHECK(RW.numel() >= X.size(1), "flashoverlap: RW must hold dim elements");
+    TORCH_CHECK(BM > 0 && BN > 0 && X.size(0) % BM == 0 && X.size(1) % BN == 0,
+                "flashoverlap: [bs, dim] must be a multiple of the tile");
+    TORCH_CHECK(RA.numel() >= (X.size(0) / BM) * (X.size(1) / BN), "flashoverlap: RA holds ", RA.numel(),
+                " entries, the matrix has ", (X.size(0) / BM) * (X.size(1) / BN), " tiles");
     check(fo_reorder_rmsnorm(dtype_of(X), dev_ptr(X, "X"), dev_ptr(RX, "RX"), dev_ptr(RW, "RW"),
                              (int)X.size(0), (int)X.size(1), (int)BM, (int)BN, (int)rldn,
                              dev_i32(RA, "RA"), (float)eps, current_stream()),
@@ -237,6 +284,8 @@ void reorder_rmsnorm(at::Tensor X, at::Tensor RX, at::Tensor RW, int64_t BM, int
 // rmsnorm, src/rmsnorm/rmsnorm.cu:32-46 (the reference compiles but does not register it).
 void rmsnorm_eps(at::Tensor X, at::Tensor O, at::Tensor RW, double eps) {
     TORCH_CHECK(X.dim() == 2 && O.sizes() == X.sizes(), "flashoverlap: X and O must be [bs, dim]");
+    TORCH_CHECK(X.scalar_type() == O.scalar_type() && X.scalar_type() == RW.scalar_type() && RW.numel() >= X.size(1),
+                "flashoverlap: X, O and RW must share one dtype and RW must hold dim elements");
     check(fo_rmsnorm(dtype_of(X), dev_ptr(X, "X"), dev_ptr(O, "O"), dev_ptr(RW, "RW"), (int)X.size(0),
                      (int)X.size(1), (float)eps, current_stream()),
           "rmsnorm");
@@ -274,7 +323,8 @@ TORCH_LIBRARY(flashoverlap_class, m) {
         .def("seg_allreduce", &OverlapImpl::seg_allreduce)
         .def("set_accumulator", &OverlapImpl::set_accumulator)
         .def("clear_accumulator", &OverlapImpl::clear_accumulator)
-        .def("set_fused_consumer", &OverlapImpl::set_fused_consumer);
+        .def("set_fused_consumer", &OverlapImpl::set_fused_consumer)
+        .def("status", &OverlapImpl::status);
 }
 
 TORCH_LIBRARY(flashoverlap_op, m) {

@@ -193,7 +193,7 @@ def measured_hint(M, N, K, algo, wave, dtype=torch.float16, warmup=20, samples=1
 
 
 def time_overlap(M, N, K, algo, cseg, hint, dtype=torch.float16, warmup=20, reps=200, fused=False,
-                 with_consumer=True):
+                 with_consumer=True, settle_s=0.2):
     """Mean ms of the overlapped call for one cSeg (tune/search.py:255-347)."""
     BM, BN = _capi.algo_tile(algo)
     TM, TN = M // BM, N // BN
@@ -209,10 +209,10 @@ def time_overlap(M, N, K, algo, cseg, hint, dtype=torch.float16, warmup=20, reps
     if with_consumer:
         ov.set_accumulator(torch.zeros(M * N, device="cuda", dtype=dtype))
     if len(cseg) == 1:
-        ms = _time_ms(lambda: ov.gemm_allreduce(A, B, C, algo), warmup, reps, settle_s=0.2)
+        ms = _time_ms(lambda: ov.gemm_allreduce(A, B, C, algo), warmup, reps, settle_s=settle_s)
     else:
         ms = _time_ms(lambda: ov.gemm_allreduce_overlap(A, B, C, MM, RA, 1, cseg_cpu, cseg_gpu, algo),
-                      warmup, reps, settle_s=0.2)
+                      warmup, reps, settle_s=settle_s)
     torch.cuda.synchronize()
     ov.close()
     return ms

@@ -33,7 +33,8 @@ enum {
     FO_ERR_ALGO = -3,     /* Algo outside [0, fo_algo_count()) */
     FO_ERR_DTYPE = -4,    /* dtype not FO_F16 / FO_BF16 */
     FO_ERR_SEGMENTS = -5, /* sum(cSeg) != tile count, G <= 0, monitor with G > TN-1 */
-    FO_ERR_STATE = -6     /* fo_overlap_* called before the matching init */
+    FO_ERR_STATE = -6,    /* fo_overlap_* called before the matching init; a launch that does not fit the device */
+    FO_ERR_LIMIT = -7     /* more groups than the static scratch of the allocation-free call holds */
 };
 
 const char *fo_error_string(int code);
@@ -91,8 +92,9 @@ int fo_gemm(int dtype, int M, int N, int K, const void *A, const void *B, void *
  * src/overlap/gemm_signal.cu:15-97 (epilogue src/overlap/gemm_with_signal.h:236-256,
  * :291-361).  RA[TM*TN], cseg_dev[G], MM[>= G; monitor: (TM+1)*TN] are device
  * int32.  Tile t is stored at slot r = RA[t] of C viewed as
- * [(M*N)/(rLDN*BN), rLDN*BN]; after the tile's stores are released at agent
- * scope, MM[group(r)] += 1; monitor: o = MM[TN-1]++, MM[TN+r] = o.
+ * [(M*N)/(rLDN*BN), rLDN*BN]; once the tile's write-through stores have been
+ * acknowledged to every wavefront of its workgroup, MM[group(r)] += 1;
+ * monitor: o = MM[TN-1]++, MM[TN+r] = o.
  * G is an extra argument (the reference reads cSeg until the prefix sum passes
  * r); it lets the library validate on the host when cseg_host != NULL. */
 int fo_gemm_signal(int dtype, int M, int N, int K, int rLDN, const int32_t *cseg_dev, int G,
@@ -108,11 +110,15 @@ int fo_gemm_scatter(int dtype, int M, int N, int K, int rLDN, const int32_t *cse
 
 /* ---- counting / wait kernel -------------------------------------------
  * Replaces kernel_wait_flag<<<1,1,0,stream>>>(expect, counter), src/wait.cuh:5-9:
- * spins (s_sleep between agent-scope acquire polls) until *counter == expect,
- * then resets it to 0.  If the environment variable FO_WAIT_MAX_POLLS is set
- * to a positive number when the library is first used, this wait (and the one
- * inside fo_wait_reduce_groups) gives up after that many polls -- a debugging
- * aid against a hung GPU; unset, the wait is unbounded like the reference's. */
+ * spins (s_sleep between relaxed agent-scope polls) until *counter == expect,
+ * then resets it to 0 with an acquiring compare-and-swap.  If the environment
+ * variable FO_WAIT_MAX_POLLS is set to a positive number when the library is
+ * first used, this wait, fo_wait_groups and the one inside
+ * fo_wait_reduce_groups give up after that many polls -- a guard against a
+ * hung GPU; unset, the wait is unbounded like the reference's.  These
+ * stand-alone entry points have nowhere to report a give-up (use
+ * fo_wait_bounded for that); the waits enqueued by the fo_overlap_* calls
+ * report it through fo_overlap_status. */
 int fo_wait(int expect, int32_t *counter, fo_stream_t stream);
 
 /* Same, but gives up after max_polls polls (0 = unbounded) and then writes 1
@@ -241,6 +247,23 @@ int fo_overlap_plan_batches(const int32_t *cseg_host, int G, int wave_tiles, int
  * (src/overlap_impl.cu:250-258); 1: always one fo_wait_reduce_groups launch
  * with the default grid; n > 1: the same with n workgroups. */
 int fo_overlap_set_fused_consumer(fo_overlap_t *h, int fused);
+/* The two thresholds of the automatic choice above (no counterpart in the
+ * reference): GEMMs below in_stream_below_flop stay on the GEMM stream, more
+ * than fused_from_groups groups get the one-launch consumer.  The defaults
+ * (6.4e10, 16) were measured on one MI355X; a negative value restores one. */
+int fo_overlap_set_schedule(fo_overlap_t *h, double in_stream_below_flop, int fused_from_groups);
+/* Bound, in polls, of every device-side wait the handle's calls enqueue
+ * (group waits, the one-launch consumer's polls, fork and join): -1 (default)
+ * takes FO_WAIT_MAX_POLLS from the environment, 0 waits without bound like
+ * src/wait.cuh:5-9. */
+int fo_overlap_set_wait_limit(fo_overlap_t *h, int64_t max_polls);
+/* Failure detection (the reference's waiter spins forever on a lost signal):
+ * synchronises both streams of the handle and stores into *gave_up whether
+ * any bounded wait enqueued since the last query ran out of polls; the kernels
+ * behind such a wait ran on incomplete data.  A non-zero answer also clears
+ * the handle's flag words, so the handle can be used again once the caller
+ * has zeroed MM. */
+int fo_overlap_status(fo_overlap_t *h, int32_t *gave_up);
 fo_stream_t fo_overlap_comm_stream(fo_overlap_t *h);
 
 /* Gemm(A,B,C,Algo), src/overlap_impl.cu:35-48. */

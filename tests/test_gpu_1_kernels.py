@@ -131,6 +131,25 @@ def test_signal_gemm_persistent_walk(fo, oracle):
     _signal_case(fo, oracle, F16, 128, 128, 4224, 4224, 64, [1] * 1089)
 
 
+@pytest.mark.parametrize("bm,bn,M,N", [(128, 256, 4224, 2048), (256, 128, 2048, 4224)])
+@pytest.mark.parametrize("dtype,K,cseg,W", [
+    (F16, 64, [264], 0),                 # one K step per tile: nothing can ride in the next tile, signalled at once
+    (F16, 192, [100, 100, 64], 0),       # three K steps: exactly the ring's depth, no steady step
+    (BF16, 1096, [8, 256], 0),           # seventeen full K steps through the dynamic-slot steady loop, then a partial one
+    (F16, 448, [132, 132], 2),           # row-mapped stores, seven K steps
+    (BF16, 64, [1] * 264, 0),            # a group per tile
+])
+def test_signal_gemm_three_slot_shapes_walk_several_tiles(fo, oracle, dtype, K, cseg, W, bm, bn, M, N):
+    """The 128x256 and 256x128 workgroup tiles run on rings of three slots.  264 tiles on 256 resident
+    workgroups (M or N is no multiple of 256, so the workgroup tile is the Algo's own): eight workgroups
+    compute a second tile, whose first stage is requested before the first tile's epilogue, whose first
+    wait leaves that epilogue's stores in flight, and from whose first K step the first tile's signal is
+    sent while younger operand loads are still outstanding."""
+    info = fo._capi.kernel_info(_algo(fo, bm, bn, swizzle=4), M, N, epilogue=2 if W else 1, dtype=dtype)
+    assert info["resident"] == 256 and info["lds_bytes"] == 3 * (128 + 256) * 64 * 2
+    _signal_case(fo, oracle, dtype, bm, bn, M, N, K, cseg, W=W, swizzle=4, seed=11 + K)
+
+
 @pytest.mark.parametrize("dtype", [F16, BF16])
 @pytest.mark.parametrize("bm,bn,M,N,K", [(128, 128, 256, 384, 8), (128, 128, 256, 384, 72),
                                          (128, 128, 384, 256, 200), (128, 128, 256, 256, 1376),

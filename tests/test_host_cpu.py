@@ -196,3 +196,110 @@ def test_same_wave_groups_share_a_launch():
     assert plan([1, 2, 3], 1000) == [(0, 3)]
     with pytest.raises(_capi.FlashOverlapError):
         plan([4, 0, 4], 8)
+
+
+def test_front_ends_refuse_undersized_buffers():
+    """MM, RA, RE and D are indexed through raw pointers by kernels that store and count through them;
+    both front ends must refuse buffers that are too small before anything is launched.  The case the
+    reference itself gets wrong: more groups than tile columns with MM sized TN (test/test.py:94)."""
+    from flashoverlap_amd import ops
+    i32 = lambda n: torch.zeros(n, dtype=torch.int32)
+    algo = _capi.find_algo(128, 128)
+    M, N = 512, 256                                   # 4 x 2 tiles
+    ok = dict(M=M, N=N, algo=algo, rLDN=1, G=8, MM=i32(8), RA=i32(8))
+    ops._check_signal_buffers(**ok)
+    for bad, what in [(dict(MM=i32(2)), "MM holds 2"),           # sized TN although G = 8
+                      (dict(MM=i32(9), monitor=True), "MM holds 9"),   # monitor needs (TM+1)*TN = 10
+                      (dict(RA=i32(6)), "RA holds 6"),
+                      (dict(rLDN=3), "rLDN"),
+                      (dict(RE=i32(1023)), "RE holds 1023"),     # M*N/BN = 1024 rows
+                      (dict(D=torch.zeros(100), W=4), "D holds 100"),
+                      (dict(M=500), "not a multiple")]:
+        with pytest.raises(ValueError, match=what):
+            ops._check_signal_buffers(**{**ok, **bad})
+    ops._check_signal_buffers(**{**ok, "RE": i32(1024), "D": torch.zeros(M * N // 4), "W": 4})
+    with pytest.raises(ValueError, match="acc holds"):
+        ops._check_rs(torch.zeros(64).half(), torch.zeros(3 * 100 + 15).half(), 4, 100)
+    ops._check_rs(torch.zeros(64).half(), torch.zeros(3 * 100 + 16).half(), 4, 100)
+    with pytest.raises(ValueError, match="own holds"):
+        ops._check_rs(torch.zeros(64).half(), torch.zeros(400).half(), 4, 100, own=torch.zeros(8).half())
+    with pytest.raises(TypeError):
+        ops._check_rs(torch.zeros(64).half(), torch.zeros(400).bfloat16(), 4, 100)
+    with pytest.raises(ValueError):
+        ops._check_norm(torch.zeros(4, 64).half(), torch.zeros(4, 32).half(), torch.zeros(64).half())
+
+    # the drop-in classes check the same things before they unpack a pointer (CPU tensors get that far)
+    from flashoverlap_amd import layers
+    layers.load_library()
+    ov = torch.classes.flashoverlap_class.OverlapImpl()
+    ov.nccl_init(0, 4, [0] * 16)
+    A, B, C = torch.zeros(M, 64).half(), torch.zeros(N, 64).half(), torch.zeros(M, N).half()
+    RA, cs = i32(8).reshape(4, 2), i32(8)
+    with pytest.raises(RuntimeError, match="MM holds 2"):
+        ov.gemm_allreduce_overlap(A, B, C, i32(2), RA, 1, cs, cs, algo, False)
+    with pytest.raises(RuntimeError, match="MM holds 9"):
+        ov.gemm_allreduce_overlap(A, B, C, i32(9), RA, 1, cs, cs, algo, True)
+    with pytest.raises(RuntimeError, match="RA must be"):
+        ov.gemm_allreduce_overlap(A, B, C, i32(8), RA.reshape(2, 4), 1, cs, cs, algo, False)
+    with pytest.raises(RuntimeError, match="RE holds"):
+        ov.gemm_reducescatter_overlap(A, B, C, torch.zeros(M // 4, N).half(), i32(8), RA, i32(100), 1, cs, cs, algo, False)
+    with pytest.raises(RuntimeError, match="D holds"):
+        ov.gemm_reducescatter_overlap(A, B, C, torch.zeros(M // 8, N).half(), i32(8), RA, i32(1024), 1, cs, cs, algo, False)
+    with pytest.raises(RuntimeError, match="RA holds"):
+        torch.ops.flashoverlap_op.reorder_rmsnorm(C, C.clone(), torch.zeros(N).half(), 128, 128, 1, i32(7))
+
+
+def test_new_handle_calls_validate_without_gpu():
+    L = _capi.lib()
+    null = ctypes.c_void_p()
+    one = ctypes.c_void_p(16)
+    h = ctypes.c_void_p()
+    assert L.fo_overlap_create(ctypes.byref(h)) == 0
+    out = ctypes.c_int32(7)
+    assert L.fo_overlap_status(h, ctypes.byref(out)) == 0 and out.value == 0    # nothing enqueued yet
+    assert L.fo_overlap_status(h, null) == -1
+    assert L.fo_overlap_set_wait_limit(h, -2) == -1 and L.fo_overlap_set_wait_limit(h, 1000) == 0
+    assert L.fo_overlap_set_schedule(h, -1.0, -1) == 0
+    assert L.fo_overlap_destroy(h) == 0
+
+
+def test_config1_checker_against_torch_cpu(oracle):
+    """BASELINE configuration 1 on the CPU: fp16 1024^3, A and B N(0,1)/sqrt(K) from seed 0, fp32 accumulate,
+    128x128 tiles, wave groups of 2 waves (a nominal wave of 8 tiles, so 16 tiles per group), reorder by
+    group, then RMSNorm over N with eps 1e-6 and gamma = 1 + 0.01 N(0,1).  The checker's whole path
+    (signal GEMM into the reordered buffer, counts, reorder+RMSNorm) against torch's CPU matmul and the
+    RMSNorm of example/RMSNorm.py:13-18."""
+    M = N = K = 1024
+    bm = bn = 128
+    g = torch.Generator().manual_seed(0)
+    A16 = (torch.randn(M, K, generator=g) * K ** -0.5).half()
+    B16 = (torch.randn(N, K, generator=g) * K ** -0.5).half()
+    gamma = (1 + 0.01 * torch.randn(N, generator=g)).half()
+    T = (M // bm) * (N // bn)
+    cseg = layout.cseg_from_waves(T, 2 * 8)
+    assert cseg == [16] * 4
+    # a simulated completion order: waves of 8 tiles walking the columns of the tile grid first
+    hint = [tm * (N // bn) + tn for tn in range(N // bn) for tm in range(M // bm)]
+    ra = layout.reorder_indices(T, hint, device="cpu").numpy()
+    bits = lambda t: t.contiguous().view(torch.int16).numpy().view(np.uint16)
+    cp, mm = oracle.gemm_signal(oracle.F16, bits(A16), bits(B16), bm, bn, RA=ra, cseg=cseg)
+    assert mm[:4].tolist() == cseg                                      # signal counts, bit-exact
+    ref = A16.float() @ B16.float().T                                   # torch CPU, fp32 accumulate
+    back = torch.from_numpy(oracle.from_bits(oracle.unpermute(cp, M, N, bm, bn, ra), oracle.F16)).reshape(M, N)
+    rel = ((back - ref).abs() / ref.abs().clamp_min(ref.abs().mean())).max().item()
+    assert rel <= 1e-2
+    assert (back.half() == ref.half()).float().mean() > 0.99            # same fp32 sums up to summation order
+    # every group's tiles are one contiguous run of the reordered buffer: group k = tile columns 2k, 2k+1
+    C16 = back.half()
+    run = torch.from_numpy(oracle.from_bits(cp, oracle.F16)).reshape(T, bm, bn)
+    for k, t in enumerate(hint):
+        tm, tn = divmod(t, N // bn)
+        assert torch.equal(run[k].half(), C16[tm * bm:(tm + 1) * bm, tn * bn:(tn + 1) * bn])
+    # reorder+RMSNorm of the reordered buffer against the reference formula on the row-major product
+    y = oracle.from_bits(oracle.reorder_rmsnorm(oracle.F16, cp, bits(gamma), M, N, bm, bn, 1, ra, eps=1e-6), oracle.F16)
+    x = C16.float()
+    want = ((x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6)).half() * gamma).float()   # RMSNorm.py:13-18
+    got = torch.from_numpy(y).reshape(M, N)
+    rel = ((got - want).abs() / want.abs().clamp_min(want.abs().mean())).max().item()
+    assert rel <= 1e-2
+    assert (got == want).float().mean() > 0.98
