@@ -60,6 +60,8 @@ SIGNATURES = {
                                               vp, c_int, c_int, c_int, vp, vp, c_int, c_int, c_int]),
     "fo_overlap_gemm_allreduce_serial": (c_int, [vp, c_int, c_int, c_int, c_int, vp, vp, vp, c_int]),
     "fo_overlap_seg_allreduce": (c_int, [vp, c_int, vp, c_i64, vp, c_int, c_int]),
+    "fo_gemm_allreduce_overlap_static": (c_int, [c_int, c_int, c_int, c_int, vp, vp, vp, vp, vp, c_int, c_int, c_int,
+                                                 vp, vp, c_int, c_int, c_int, vp, vp]),
 }
 
 _lib = None

@@ -146,6 +146,7 @@ extern "C" const char *fo_error_string(int code) {
         case FO_ERR_DTYPE: return "dtype must be FO_F16 or FO_BF16";
         case FO_ERR_SEGMENTS: return "cSeg does not partition the tiles (or too many groups for monitor mode)";
         case FO_ERR_STATE: return "fo_overlap handle used before its init call, or a launch that does not fit this device";
+        case FO_ERR_LIMIT: return "more groups than the static scratch of the allocation-free call holds (4096)";
         default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
     }
 }

@@ -500,3 +500,79 @@ extern "C" int fo_overlap_seg_allreduce(fo_overlap_t *h, int dtype, void *C, int
     }
     return FO_OK;
 }
+
+// ---------------------------------------------------------------- handle-free call that allocates nothing
+// Callers that cannot allocate (code under a harness that forbids it, serving
+// loops) have no handle: a handle owns a hipMalloc'ed workspace and, in the
+// reference's interface, the caller brings the counters MM in a tensor of its own.
+// Here both live in this file-scope array: kWorkspaceWords flag words, then one
+// counter per group.  Each device the library runs on holds its own copy until the
+// process ends; its address is asked for once per device.
+constexpr int kStaticMaxGroups = 4096;
+static __device__ __align__(256) int32_t scratch[kWorkspaceWords + kStaticMaxGroups];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+int32_t *g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each device (the array's name is not one)
+int g_scratch_token[kMaxDevices];     // last fork/join token handed out on each device
+
+int scratch_of_current_device(int32_t **ptr, int *token) {
+    int dev = 0;
+    FO_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return FO_ERR_STATE;
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        FO_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return FO_ERR_STATE;
+        g_scratch_ptr[dev] = static_cast<int32_t *>(p);
+    }
+    *ptr = g_scratch_ptr[dev];
+    // never 0 (the words' resting value) and never the previous call's, so a word
+    // that an abandoned wait left behind cannot pass for this call's
+    g_scratch_token[dev] = g_scratch_token[dev] >= (1 << 30) ? 1 : g_scratch_token[dev] + 1;
+    *token = g_scratch_token[dev];
+    return FO_OK;
+}
+
+}  // namespace
+
+extern "C" int fo_gemm_allreduce_overlap_static(int dtype, int M, int N, int K, const void *A, const void *B,
+                                                void *C, void *acc, const int32_t *RA, int TM, int TN, int rLDN,
+                                                const int32_t *cseg_host, const int32_t *cseg_dev, int G, int algo,
+                                                int fused, fo_stream_t gemm_stream, fo_stream_t comm_stream) {
+    if (G > kStaticMaxGroups) return FO_ERR_LIMIT;
+    if (G <= 0 || !cseg_host || !cseg_dev) return FO_ERR_SEGMENTS;
+    int32_t *ws = nullptr;
+    int token = 0;
+    int rc = scratch_of_current_device(&ws, &token);
+    if (rc) return rc;
+    fo_overlap ctx;
+    ctx.gemm_stream = static_cast<hipStream_t>(gemm_stream);
+    ctx.comm_stream = comm_stream == gemm_stream ? nullptr : static_cast<hipStream_t>(comm_stream);
+    ctx.workspace = ws;
+    ctx.gemm_ready = ctx.overlap_ready = true;
+    ctx.acc = acc;
+    ctx.acc_nelem = acc ? (int64_t)M * N : 0;
+    ctx.fused = fused < 0 ? -1 : fused;
+    ctx.token = token;
+    ctx.always_fork = true;
+    // Validate before the first launch, so that a refused call leaves nothing enqueued.
+    int32_t info[12];
+    rc = fo_algo_info(algo, info);
+    if (rc) return rc;
+    if (M <= 0 || N <= 0 || M % info[0] || N % info[1] || TM != M / info[0] || TN != N / info[1]) return FO_ERR_SHAPE;
+    rc = check_segments(cseg_host, G, (long)TM * TN);
+    if (rc) return rc;
+    if (!A || !B || !C || !RA || K <= 0 || K % 8) return !A || !B || !C || !RA || K <= 0 ? FO_ERR_ARG : FO_ERR_SHAPE;
+    if (ctx.comm_stream && capturing(&ctx)) return FO_ERR_STATE;  // two streams under capture need the handle's events
+    // The array keeps what the last call on this device left: counters of a call whose
+    // bounded wait gave up would still be standing.  Cleared by a kernel, not a memset
+    // node, in case the GEMM stream is being captured.
+    rc = fo_fill_words(ws, kWorkspaceWords + G, 0, ctx.gemm_stream);
+    if (rc) return rc;
+    return allreduce_overlap(&ctx, dtype, M, N, K, A, B, C, ws + kWorkspaceWords, RA, TM, TN, rLDN, cseg_host,
+                             cseg_dev, G, algo, 0);
+}

@@ -303,3 +303,27 @@ class Overlap:
                                              cseg_cpu.numel(), int(seg_num)),
               "fo_overlap_seg_allreduce")
 
+
+def gemm_allreduce_overlap_static(A, B, C, acc, RA, rLDN, cseg_cpu, cseg_gpu, algo, fused=-1, gemm_stream=None,
+                                  comm_stream=None):
+    """fo_gemm_allreduce_overlap_static: the overlapped all-reduce call without a handle and without MM;
+    counters and flag words live in the library's static device array, nothing is allocated.
+    comm_stream None keeps the call on the GEMM stream."""
+    M, N, K = _mnk(A, B, C)
+    if RA.dim() != 2:
+        raise ValueError("RA must be [TM, TN]")
+    bm, bn = _capi.algo_tile(algo)
+    if M % bm or N % bn or RA.numel() != (M // bm) * (N // bn):
+        raise ValueError("RA does not match the Algo's tiling of M x N")
+    if cseg_cpu.numel() != cseg_gpu.numel():
+        raise ValueError("cSEG_CPU and cSEG_GPU differ in length")
+    _same_dtype(A, acc)
+    if acc is not None and acc.numel() < M * N:
+        raise ValueError(f"the accumulator holds {acc.numel()} elements, M*N = {M * N}")
+    TM, TN = RA.shape
+    gs = _stream(gemm_stream)
+    cs = gs if comm_stream is None else _stream(comm_stream)
+    check(lib().fo_gemm_allreduce_overlap_static(
+        dtype_code(A), M, N, K, _ptr(A, "A"), _ptr(B, "B"), _ptr(C, "C"), _ptr(acc, "ACC"), _i32(RA, "RA"), TM, TN,
+        int(rLDN), _i32(cseg_cpu, "cSEG_CPU", cuda=False), _i32(cseg_gpu, "cSEG_GPU"), cseg_gpu.numel(), int(algo),
+        int(fused), gs, cs), "fo_gemm_allreduce_overlap_static")

@@ -296,6 +296,29 @@ int fo_overlap_gemm_allreduce_serial(fo_overlap_t *h, int dtype, int M, int N, i
 int fo_overlap_seg_allreduce(fo_overlap_t *h, int dtype, void *C, int64_t MN,
                              const int32_t *cseg_host, int G, int seg_num);
 
+/* ---- allocation-free call ------------------------------------------------
+ * No counterpart in the reference.  For callers that cannot allocate device
+ * memory or create a handle: code running under a harness that forbids
+ * hipMalloc, tight serving loops, code inside a stream capture.  It is
+ * fo_overlap_gemm_allreduce without the handle and without MM: the group
+ * counters and the flag words of fork, join and the one-launch consumer live
+ * in a static device array inside the library (16 + 4096 int32 per device,
+ * held until the process ends), the streams and the accumulator come as
+ * arguments, and nothing is allocated, freed or created -- no hipMalloc, no
+ * stream, no event.  acc may be NULL (no consumer), comm_stream == gemm_stream
+ * keeps the whole call on one stream (the only form that can be captured into
+ * a graph: two streams under capture return FO_ERR_STATE).  fused as in
+ * fo_overlap_set_fused_consumer.  G > 4096 returns FO_ERR_LIMIT; the monitor is
+ * not available (its stamps are an output that needs a caller's buffer).
+ * The array is cleared by a small kernel at the start of every call.  All
+ * calls on one device share it: two calls that overlap in time on one device
+ * (different stream pairs, different host threads) race on the counters;
+ * calls on the same stream pair are ordered by the join and do not. */
+int fo_gemm_allreduce_overlap_static(int dtype, int M, int N, int K, const void *A, const void *B, void *C,
+                                     void *acc, const int32_t *RA, int TM, int TN, int rLDN,
+                                     const int32_t *cseg_host, const int32_t *cseg_dev, int G, int algo,
+                                     int fused, fo_stream_t gemm_stream, fo_stream_t comm_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -261,6 +261,12 @@ def test_new_handle_calls_validate_without_gpu():
     assert L.fo_overlap_set_wait_limit(h, -2) == -1 and L.fo_overlap_set_wait_limit(h, 1000) == 0
     assert L.fo_overlap_set_schedule(h, -1.0, -1) == 0
     assert L.fo_overlap_destroy(h) == 0
+    assert b"4096" in L.fo_error_string(-7)
+    # the allocation-free call validates before it touches a device: too many groups for its static counters
+    assert L.fo_gemm_allreduce_overlap_static(0, 128, 128, 64, one, one, one, null, one, 1, 1, 1, one, one, 4097, 0,
+                                              -1, null, null) == -7
+    assert L.fo_gemm_allreduce_overlap_static(0, 128, 128, 64, one, one, one, null, one, 1, 1, 1, null, one, 1, 0,
+                                              -1, null, null) == -5
 
 
 def test_config1_checker_against_torch_cpu(oracle):
