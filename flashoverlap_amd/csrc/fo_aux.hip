@@ -2,6 +2,8 @@
 // consumer that stands in for the collective, and (reorder+)RMSNorm.
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "fo_common.h"
 
 namespace {
@@ -304,118 +306,202 @@ __global__ __launch_bounds__(CONSUMER_THREADS, 8) void fo_wait_reduce_kernel(
 }
 
 // ------------------------------------------------------------------ RMSNorm
+// Per-dtype arithmetic on one 16-byte chunk (8 elements).
+//   sumsq: acc + sum of squares, fp32 (v_dot2c_f32_{f16,bf16}: two elements per instruction).
+//   scale: y = round16(round16(x*s) * w), the two roundings of src/rmsnorm/rmsnorm.cuh:109-113.
+//          The second product is a 16-bit multiply in the reference; the exact product of two
+//          16-bit values rounded once is the same number, so fp16 uses the packed 16-bit
+//          multiply and bf16 (no packed arithmetic on this part) an fp32 multiply and one rounding.
+template <typename Tag> struct norm_math;
+template <> struct norm_math<fo_f16_tag> {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ float sumsq(fo_u32x4 v, float acc) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint32_t u = v[k];  // a copy: the cast must see this element, not the vector's first
+            const h2 p = __builtin_bit_cast(h2, u);
+            acc = __builtin_amdgcn_fdot2(p, p, acc, false);
+        }
+        return acc;
+    }
+    static __device__ __forceinline__ fo_u32x4 scale(fo_u32x4 v, float s, fo_u32x4 w) {
+        fo_u32x4 o;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint32_t u = v[k], uw = w[k];
+            const h2 p = __builtin_bit_cast(h2, u);
+            h2 q;
+            q.x = (_Float16)((float)p.x * s);
+            q.y = (_Float16)((float)p.y * s);
+            const h2 y = q * __builtin_bit_cast(h2, uw);
+            o[k] = __builtin_bit_cast(uint32_t, y);
+        }
+        return o;
+    }
+};
+template <> struct norm_math<fo_bf16_tag> {
+    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+    typedef fo_elem<fo_bf16_tag> E;
+    static __device__ __forceinline__ float sumsq(fo_u32x4 v, float acc) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint32_t u = v[k];
+            const b2 p = __builtin_bit_cast(b2, u);
+            acc = __builtin_amdgcn_fdot2_f32_bf16(p, p, acc, false);
+        }
+        return acc;
+    }
+    static __device__ __forceinline__ fo_u32x4 scale(fo_u32x4 v, float s, fo_u32x4 w) {
+        fo_u32x4 o;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint32_t u = v[k], uw = w[k];
+            const float lo = E::to_f32(E::from_f32(E::to_f32((uint16_t)(u & 0xffff)) * s));
+            const float hi = E::to_f32(E::from_f32(E::to_f32((uint16_t)(u >> 16)) * s));
+            const uint16_t ylo = E::from_f32(lo * E::to_f32((uint16_t)(uw & 0xffff)));
+            const uint16_t yhi = E::from_f32(hi * E::to_f32((uint16_t)(uw >> 16)));
+            o[k] = (uint32_t)ylo | ((uint32_t)yhi << 16);
+        }
+        return o;
+    }
+};
+
 // One wavefront per output row, four rows per workgroup; each lane keeps its
 // 16-byte chunks of the row in registers between the sum of squares and the
-// scaling, so the row is read once.  With RA != nullptr the chunks are gathered
-// from the tile-reordered buffer (index math of src/rmsnorm/rmsnorm.cuh:80-86).
+// scaling, so the row is read once.  How a chunk's source address is found:
+//   NORM_PLAIN    the row itself (no reorder table);
+//   NORM_SLOTS    gathered from the tile-reordered buffer with rldn == 1, BN a power of
+//                 two and at most 128 tiles per row (every tile of the Algo table up to
+//                 16384 columns): tile r is the contiguous block of BM rows of BN columns
+//                 that starts at row r * BM, the index math is shifts and masks, and the
+//                 storage slots of the row's tiles are fetched once per wavefront (lane l
+//                 holds the slots of tiles l and l + 64) and handed out by shuffles: a
+//                 table load per chunk would put a second memory round trip in front of
+//                 every load of the row;
+//   NORM_GENERAL  the index math of src/rmsnorm/rmsnorm.cuh:80-86 as written (divisions,
+//                 a table load per chunk, batched in front of the row's loads).
+// The path is a template parameter so that the loop that requests the row holds no
+// branch: all of a row's loads are in flight before the first is waited for (with the
+// paths as run-time branches inside that loop every chunk waited for its own load,
+// sixteen round trips per row of 8192).  Lanes beyond the row's end request the row's
+// last chunk again and are masked out of the sum and the stores.
 // The second launch bound caps the registers (128 up to 16 chunks per lane, 256 above) so that
 // enough wavefronts stay resident to cover the memory latency.
 // STREAM: rows are read and written with non-temporal accesses (matrices that do not fit
 // into the memory-side cache beside the GEMM's operands: inside the overlapped step the
 // 8192x8192 RMSNorm then takes 55 instead of 64 us, and the GEMM that follows it 3 % less).
-template <typename Tag, int MAXCH, bool STREAM>
+enum { NORM_PLAIN = 0, NORM_SLOTS = 1, NORM_GENERAL = 2 };
+
+template <typename Tag, int MAXCH, bool STREAM, int PATH>
 __global__ __launch_bounds__(256, MAXCH <= 16 ? 4 : 2) void fo_rmsnorm_kernel(const fo_u32x4 *X, fo_u32x4 *Y, const fo_u32x4 *Wt,
                                                          int bs, int dim, int BM, int BN, int rldn,
                                                          const int32_t *RA, float eps) {
-    typedef fo_elem<Tag> E;
+    typedef norm_math<Tag> MATH;
+    // The weight goes through LDS, fetched once per workgroup ahead of the rows: a weight
+    // load from memory between two stores of the output row would make its wait (vmcnt
+    // retires in order) a wait for the store before it, one round trip per chunk.
+    __shared__ fo_u32x4 wlds[64 * MAXCH];
     const int lane = threadIdx.x & 63;
-    const int b = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (b >= bs) return;
     const int nch = dim >> 3;  // 16-byte chunks per row
-    const int ldn = RA ? dim / BN : 0;
-    const int tile_row = RA ? b / BM : 0, in_row = RA ? b % BM : 0;
-    const long ldp16 = RA ? ((long)rldn * BN) >> 3 : 0;
-    const int bn_shift = (RA && rldn == 1 && (BN & (BN - 1)) == 0) ? __builtin_ctz(BN) : -1;
-
-    // The storage slots of this row's tiles, fetched once per wavefront (lane l holds the
-    // slots of tiles l and l + 64) and handed out by shuffles: a table load per chunk would
-    // put a second memory round trip in front of every load of the row (measured with
-    // nothing cached, 8192 x 8192: 69 us against 52 us for the plain RMSNorm).
-    const bool slots_in_lanes = bn_shift >= 0 && ldn <= 128;
-    int slot_lo = 0, slot_hi = 0;
-    if (slots_in_lanes) {
-        const int32_t *row = RA + (long)tile_row * ldn;
-        if (lane < ldn) slot_lo = row[lane];
-        if (lane + 64 < ldn) slot_hi = row[lane + 64];
+    constexpr int WPT = MAXCH / 4;  // weight chunks per lane of the workgroup
+    fo_u32x4 wreg[WPT];
+#pragma unroll
+    for (int q = 0; q < WPT; q++) {
+        const int c = threadIdx.x + q * 256;
+        wreg[q] = Wt[c < nch ? c : nch - 1];
     }
+    const int b = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const bool live = b < bs;  // a workgroup's rows beyond the matrix: the wavefront only helps with the weight
+    const bool full = nch == 64 * MAXCH;  // every lane owns MAXCH chunks of the row
+    const int ldn = PATH == NORM_PLAIN ? 0 : dim / BN;
+    const int row_b = live ? b : bs - 1;  // such a wavefront requests the last row again and discards it
+    const int tile_row = PATH == NORM_PLAIN ? 0 : row_b / BM, in_row = PATH == NORM_PLAIN ? 0 : row_b % BM;
+    auto chunk_of = [&](int i) {  // this lane's i-th chunk, clamped into the row
+        const int c = lane + i * 64;
+        return c < nch ? c : nch - 1;
+    };
+    auto fetch = [&](long src) -> fo_u32x4 { return STREAM ? __builtin_nontemporal_load(&X[src]) : X[src]; };
 
     fo_u32x4 x[MAXCH];
+    if (PATH == NORM_PLAIN) {
+#pragma unroll
+        for (int i = 0; i < MAXCH; i++) x[i] = fetch((long)row_b * nch + chunk_of(i));
+    } else if (PATH == NORM_SLOTS) {
+        const int bn_shift = __builtin_ctz(BN);
+        const int32_t *row = RA + (long)tile_row * ldn;
+        const int slot_lo = lane < ldn ? row[lane] : 0;
+        auto request = [&](auto two_regs) {
+            int slot_hi = 0;
+            if (decltype(two_regs)::value) slot_hi = lane + 64 < ldn ? row[lane + 64] : 0;
+#pragma unroll
+            for (int i = 0; i < MAXCH; i++) {
+                const int j = chunk_of(i) << 3;
+                const int t = j >> bn_shift;
+                int r = __shfl(slot_lo, t & 63, 64);
+                if (decltype(two_regs)::value) {
+                    const int hi = __shfl(slot_hi, t & 63, 64);
+                    r = t < 64 ? r : hi;
+                }
+                x[i] = fetch((((long)r * BM + in_row) << (bn_shift - 3)) + ((j & (BN - 1)) >> 3));
+            }
+        };
+        if (ldn <= 64)
+            request(std::false_type{});
+        else
+            request(std::true_type{});
+    } else {
+        const long ldp16 = ((long)rldn * BN) >> 3;
+        int r[MAXCH];
+#pragma unroll
+        for (int i = 0; i < MAXCH; i++) r[i] = RA[tile_row * ldn + (chunk_of(i) << 3) / BN];
+#pragma unroll
+        for (int i = 0; i < MAXCH; i++) {
+            const int j = chunk_of(i) << 3;
+            const long nr = (long)(r[i] / rldn) * BM + in_row;
+            const int nc = (r[i] % rldn) * BN + j % BN;
+            x[i] = fetch(nr * ldp16 + (nc >> 3));
+        }
+    }
+
+    // the weight chunks were requested before the row: they are in registers when the row's
+    // first chunk is (in-order return)
+#pragma unroll
+    for (int q = 0; q < WPT; q++) wlds[threadIdx.x + q * 256] = wreg[q];
+
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < MAXCH; i++) {
-        const int c = lane + i * 64;
-        // shuffles are executed by all lanes; chunks beyond the row ask for tile 0
-        int r_lanes = 0;
-        if (slots_in_lanes) {
-            const int t = c < nch ? (c << 3) >> bn_shift : 0;
-            const int lo = __shfl(slot_lo, t & 63, 64), hi = __shfl(slot_hi, t & 63, 64);
-            r_lanes = t < 64 ? lo : hi;
-        }
-        if (c < nch) {
-            long src;
-            if (RA) {
-                const int j = c << 3;
-                if (slots_in_lanes) {
-                    // rldn == 1 and BN a power of two (every tile of the Algo table): tile r is
-                    // the contiguous block of BM rows of BN columns that starts at row r * BM
-                    src = ((long)r_lanes * BM + in_row) * ldp16 + ((j & (BN - 1)) >> 3);
-                } else if (bn_shift >= 0) {
-                    const int r = RA[tile_row * ldn + (j >> bn_shift)];
-                    src = ((long)r * BM + in_row) * ldp16 + ((j & (BN - 1)) >> 3);
-                } else {
-                    const int r = RA[tile_row * ldn + j / BN];
-                    const long nr = (long)(r / rldn) * BM + in_row;
-                    const int nc = (r % rldn) * BN + j % BN;
-                    src = nr * ldp16 + (nc >> 3);
-                }
-            } else {
-                src = (long)b * nch + c;
-            }
-            x[i] = STREAM ? __builtin_nontemporal_load(&X[src]) : X[src];
-            const uint32_t w[4] = {x[i].x, x[i].y, x[i].z, x[i].w};
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                const float lo = E::to_f32((uint16_t)(w[k] & 0xffff));
-                const float hi = E::to_f32((uint16_t)(w[k] >> 16));
-                ss += lo * lo;
-                ss += hi * hi;
-            }
-        }
+        const float with = MATH::sumsq(x[i], ss);
+        ss = (full || lane + i * 64 < nch) ? with : ss;
     }
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) ss += __shfl_xor(ss, d, 64);
     const float s = rsqrtf(ss / (float)dim + eps);
+    __syncthreads();  // the weight is in LDS
+    if (!live) return;
 
+    fo_u32x4 *out = Y + (long)b * nch;
+    auto emit = [&](auto whole_row) {
 #pragma unroll
-    for (int i = 0; i < MAXCH; i++) {
-        const int c = lane + i * 64;
-        if (c < nch) {
-            const fo_u32x4 wv = Wt[c];
-            const uint32_t xi[4] = {x[i].x, x[i].y, x[i].z, x[i].w};
-            const uint32_t wi[4] = {wv.x, wv.y, wv.z, wv.w};
-            uint32_t o[4];
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                // y = round16(round16(x*s) * w): the second product is a 16-bit
-                // multiply in the reference (rmsnorm.cuh:110-112); the fp32
-                // product of two 16-bit values is exact, so one rounding matches.
-                const float lo = E::to_f32(E::from_f32(E::to_f32((uint16_t)(xi[k] & 0xffff)) * s));
-                const float hi = E::to_f32(E::from_f32(E::to_f32((uint16_t)(xi[k] >> 16)) * s));
-                const uint16_t ylo = E::from_f32(lo * E::to_f32((uint16_t)(wi[k] & 0xffff)));
-                const uint16_t yhi = E::from_f32(hi * E::to_f32((uint16_t)(wi[k] >> 16)));
-                o[k] = (uint32_t)ylo | ((uint32_t)yhi << 16);
+        for (int i = 0; i < MAXCH; i++) {
+            const int c = lane + i * 64;
+            if (decltype(whole_row)::value || c < nch) {
+                const fo_u32x4 y = MATH::scale(x[i], s, wlds[c]);
+                if (STREAM)
+                    __builtin_nontemporal_store(y, &out[c]);
+                else
+                    out[c] = y;
             }
-            const fo_u32x4 y = {o[0], o[1], o[2], o[3]};
-            if (STREAM)
-                __builtin_nontemporal_store(y, &Y[(long)b * nch + c]);
-            else
-                Y[(long)b * nch + c] = y;
         }
-    }
+    };
+    if (full)
+        emit(std::true_type{});
+    else
+        emit(std::false_type{});
 }
 
-template <typename Tag, bool STREAM>
-int launch_rmsnorm_as(const void *X, void *Y, const void *Wt, int bs, int dim, int BM, int BN,
+template <typename Tag, bool STREAM, int PATH>
+int launch_rmsnorm_on(const void *X, void *Y, const void *Wt, int bs, int dim, int BM, int BN,
                       int rldn, const int32_t *RA, float eps, hipStream_t stream) {
     const int nch = dim / 8;
     dim3 grid((bs + 3) / 4), block(256);
@@ -423,17 +509,26 @@ int launch_rmsnorm_as(const void *X, void *Y, const void *Wt, int bs, int dim, i
     fo_u32x4 *y = static_cast<fo_u32x4 *>(Y);
     const fo_u32x4 *w = static_cast<const fo_u32x4 *>(Wt);
     if (nch <= 64 * 4)
-        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 4, STREAM>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
+        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 4, STREAM, PATH>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
     else if (nch <= 64 * 8)
-        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 8, STREAM>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
+        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 8, STREAM, PATH>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
     else if (nch <= 64 * 16)
-        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 16, STREAM>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
+        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 16, STREAM, PATH>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
     else if (nch <= 64 * 32)
-        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 32, STREAM>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
+        hipLaunchKernelGGL((fo_rmsnorm_kernel<Tag, 32, STREAM, PATH>), grid, block, 0, stream, x, y, w, bs, dim, BM, BN, rldn, RA, eps);
     else
         return FO_ERR_SHAPE;  // rows above 16384 elements (the reference's limit too)
     FO_LAUNCH_CHECK();
     return FO_OK;
+}
+
+template <typename Tag, bool STREAM>
+int launch_rmsnorm_as(const void *X, void *Y, const void *Wt, int bs, int dim, int BM, int BN,
+                      int rldn, const int32_t *RA, float eps, hipStream_t stream) {
+    if (!RA) return launch_rmsnorm_on<Tag, STREAM, NORM_PLAIN>(X, Y, Wt, bs, dim, BM, BN, rldn, RA, eps, stream);
+    if (rldn == 1 && (BN & (BN - 1)) == 0 && dim / BN <= 128)
+        return launch_rmsnorm_on<Tag, STREAM, NORM_SLOTS>(X, Y, Wt, bs, dim, BM, BN, rldn, RA, eps, stream);
+    return launch_rmsnorm_on<Tag, STREAM, NORM_GENERAL>(X, Y, Wt, bs, dim, BM, BN, rldn, RA, eps, stream);
 }
 
 template <typename Tag>
