@@ -23,7 +23,7 @@ PEAK_TFLOPS = 2516.6   # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the signal GEMM, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
 # profiles/gemm_c5_hbm_traffic.md (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 256 MiB copy).
-MEASURED_TRAFFIC_BYTES = {("c5", "f16"): 879432.6 * 1024 * 2.0 + 131136.0 * 1024}
+MEASURED_TRAFFIC_BYTES = {("c5", "f16"): 838479.1 * 1024 * 2.0 + 131136.0 * 1024}
 
 WORKLOADS = {
     # name: (M, N, K, BM, BN, dtype, group tiles, W, description)
