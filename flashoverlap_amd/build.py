@@ -32,12 +32,17 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
 
 KERNEL_SOURCES = ["fo_gemm.hip", "fo_aux.hip", "fo_algo.cpp", "fo_overlap.cpp"]
+# fo_gemm256_inst.hip holds one instantiation of the 256x256 GEMM kernel per compilation
+# (dtype fp16 / bf16 x plain / signal / scatter epilogue); each takes minutes, so they are separate jobs.
+GEMM256_INSTANCES = [(d, m) for d in (0, 1) for m in (0, 1, 2)]
 
 # -packed-fp32-ops off: hipcc must not form v_pk_*_f32 from the float code here.
 HIP_FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-x", "hip",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # the K step of the 256x256 kernel is one fully unrolled body of 128 MFMAs built from nested constant loops
+    "-mllvm", "-pragma-unroll-threshold=1000000",
     "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
 ]
 
@@ -53,13 +58,18 @@ def _run(cmd):
 def build_kernels(extra_flags=()):
     os.makedirs(OBJDIR, exist_ok=True)
 
-    def compile_one(src):
-        obj = os.path.join(OBJDIR, os.path.splitext(src)[0] + ".o")
-        _run([HIPCC] + HIP_FLAGS + list(extra_flags) + ["-c", os.path.join(CSRC, src), "-o", obj])
+    def compile_one(job):
+        src, defs, tag = job
+        obj = os.path.join(OBJDIR, os.path.splitext(src)[0] + tag + ".o")
+        _run([HIPCC] + HIP_FLAGS + list(extra_flags) + defs + ["-c", os.path.join(CSRC, src), "-o", obj])
         return obj
 
-    with ThreadPoolExecutor(max_workers=4) as pool:
-        objs = list(pool.map(compile_one, KERNEL_SOURCES))
+    # the long jobs first
+    jobs = [("fo_gemm256_inst.hip", [f"-DFO_INST_DTYPE={d}", f"-DFO_INST_MODE={m}"], f"_{d}_{m}")
+            for d, m in GEMM256_INSTANCES]
+    jobs += [(src, [], "") for src in KERNEL_SOURCES]
+    with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 4)) as pool:
+        objs = list(pool.map(compile_one, jobs))
     _run([HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", KERNEL_LIB] + objs)
     return KERNEL_LIB
 

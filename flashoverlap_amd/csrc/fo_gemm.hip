@@ -1,79 +1,49 @@
 // Host side of the gfx950 MFMA GEMM: picks the kernel shape for a problem and
 // launches it (plain, signal and scatter epilogues).  The device code is in
-// fo_gemm_kernel.h.
+// fo_gemm_kernel.h and fo_gemm256_kernel.h; the latter's six instantiations are
+// compiled in translation units of their own (fo_gemm256_inst.hip).
 #include <atomic>
-#include <mutex>
 
 #include "fo_gemm_kernel.h"
+#include "fo_gemm_launch.h"
 
 namespace {
 
 using namespace fo_gemm_dev;
 
-constexpr int kMaxDevices = 64;
+}  // namespace
 
-// One compiled shape of the kernel template.  The launch is persistent: as many
-// workgroups as the device keeps resident at once (or fewer, if the problem has
-// fewer macro tiles); each walks the raster with that stride.
-// With `resident_out` set nothing is launched: the call only reports how many workgroups the
-// launch would hold, in resident_out[1..3] the kernel's registers per lane, LDS bytes and
-// threads per workgroup, and in resident_out[4] how many workgroups stay resident at most.
-// expect_resident > 0: refuse (FO_ERR_STATE) unless that many stay resident.
-template <typename Tag, int MTM, int MTN, int BK, int SA, int SB, int WM, int WN, int MODE>
-int launch_variant(const GemmArgs &a, hipStream_t stream, int *resident_out, int expect_resident) {
-    auto kern = fo_gemm_kernel<Tag, MTM, MTN, BK, SA, SB, WM, WN, MODE>;
-    constexpr int smem = smem_bytes<MTM, MTN, BK, SA, SB>();
-    constexpr int threads = WM * WN * 64;
-    // Resident workgroups of this instantiation per device; the LDS attribute is set once per device too.
-    static std::mutex mu;
-    static int resident_of[kMaxDevices];
-    int dev = 0;
-    FO_HIP_CHECK(hipGetDevice(&dev));
-    if (dev < 0 || dev >= kMaxDevices) return FO_ERR_STATE;
-    int resident;
-    {
-        std::lock_guard<std::mutex> lock(mu);
-        if (!resident_of[dev]) {
-            FO_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-            int cus = 0, per_cu = 0;
-            FO_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-            FO_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(kern),
-                                                                      threads, smem));
-            if (cus <= 0 || per_cu <= 0) return FO_ERR_STATE;
-            // a multiple of 8 keeps "workgroup id mod 8 = XCD" true for every tile of the walk
-            int r = (cus * per_cu) / 8 * 8;
-            resident_of[dev] = r > 0 ? r : cus * per_cu;
-        }
-        resident = resident_of[dev];
+int fo_gemm_dev::fo_gemm256_launch(int dtype, int mode, const GemmArgs &a, hipStream_t stream, int *resident_out,
+                                   int expect_resident) {
+    const int key = (dtype == FO_BF16 ? 3 : 0) + mode;
+    switch (key) {
+        case 0: return fo_gemm256_launch_0_0(a, stream, resident_out, expect_resident);
+        case 1: return fo_gemm256_launch_0_1(a, stream, resident_out, expect_resident);
+        case 2: return fo_gemm256_launch_0_2(a, stream, resident_out, expect_resident);
+        case 3: return fo_gemm256_launch_1_0(a, stream, resident_out, expect_resident);
+        case 4: return fo_gemm256_launch_1_1(a, stream, resident_out, expect_resident);
+        case 5: return fo_gemm256_launch_1_2(a, stream, resident_out, expect_resident);
     }
-    // The raster (and with it the schedule order handed to the caller as the hint) was laid out for
-    // expect_resident workgroups; a launch that would hold another number walks the tiles differently.
-    if (expect_resident > 0 && resident != expect_resident) return FO_ERR_STATE;
-    const int ntiles = a.count;
-    if (resident_out) {
-        hipFuncAttributes attr;
-        FO_HIP_CHECK(hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(kern)));
-        resident_out[0] = ntiles < resident ? ntiles : resident;
-        resident_out[1] = attr.numRegs;
-        resident_out[2] = smem;
-        resident_out[3] = threads;
-        resident_out[4] = resident;
-        return FO_OK;
-    }
-    dim3 grid(ntiles < resident ? ntiles : resident), block(threads);
-    hipLaunchKernelGGL(kern, grid, block, smem, stream, a);
-    FO_LAUNCH_CHECK();
-    return FO_OK;
+    return FO_ERR_ARG;
 }
 
-// Macro tile -> kernel shape.  256x256 (eight wavefronts, two 64 KiB slots of a K step's A and B
-// parts) is the workhorse; the smaller shapes (three slots for 128x256 and 256x128, two for 128x128)
-// serve problems whose M or N is not a multiple of 256 or that have too few 256x256 tiles to fill the chip.
+namespace {
+
+template <typename Tag, int MTM, int MTN, int BK, int SA, int SB, int WM, int WN, int MODE>
+int launch_variant(const GemmArgs &a, hipStream_t stream, int *resident_out, int expect_resident) {
+    return launch_kernel<fo_gemm_kernel<Tag, MTM, MTN, BK, SA, SB, WM, WN, MODE>, smem_bytes<MTM, MTN, BK, SA, SB>(),
+                         WM * WN * 64>(a, stream, resident_out, expect_resident);
+}
+
+// Macro tile -> kernel.  256x256 (fo_gemm256_kernel.h: four wavefronts of 128x128, two 64 KiB slots) is
+// the workhorse; the smaller shapes (fo_gemm_kernel.h: three slots for 128x256 and 256x128, two for
+// 128x128) serve problems whose M or N is not a multiple of 256 or that have too few 256x256 tiles to
+// fill the chip.
 template <typename Tag, int MODE>
 int launch_tile(const GemmArgs &a, int mtm, int mtn, hipStream_t stream, int *resident_out, int expect_resident) {
     if (mtm == 256 && mtn == 256)
-        return launch_variant<Tag, 256, 256, 64, 2, 2, 2, 4, MODE>(a, stream, resident_out, expect_resident);
+        return fo_gemm256_launch(std::is_same<Tag, fo_bf16_tag>::value ? FO_BF16 : FO_F16, MODE, a, stream, resident_out,
+                                 expect_resident);
     if (mtm == 128 && mtn == 128)
         return launch_variant<Tag, 128, 128, 64, 2, 2, 2, 2, MODE>(a, stream, resident_out, expect_resident);
     if (mtm == 128 && mtn == 256)
@@ -102,6 +72,7 @@ int run_gemm(int mode, int dtype, int M, int N, int K, int rLDN, const int32_t *
     int rc = fo_pick_raster(algo, M, N, &r);
     if (rc) return rc;
     if (K % 8) return FO_ERR_SHAPE;  // operand rows are fetched in 16-byte chunks
+    if (K > (1 << 21)) return FO_ERR_SHAPE;  // 256 operand rows are addressed through one 31-bit buffer range
     // the epilogue assumes a wavefront's 128 x 64 (or 64 x 64) block lies inside one reorder tile
     if (e->f[0] % 128 || e->f[1] % 128) return FO_ERR_ALGO;
     GemmArgs a;

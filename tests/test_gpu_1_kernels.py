@@ -377,14 +377,18 @@ def test_reorder_rmsnorm_undoes_the_permutation(fo, oracle, dtype):
 
 @pytest.mark.parametrize("dtype", [F16, BF16])
 def test_gemm_leaves_registers_for_a_consumer_wavefront(fo, dtype):
-    """The consumer kernels are built for one 64-register wavefront per SIMD beside the two
-    wavefronts of a signalling GEMM workgroup: 2 x GEMM registers (allocated in eights) + 64 must
-    fit the 512 of a SIMD, or the overlapped path silently degrades into a serial one."""
-    algo = _algo(fo, 128, 256, swizzle=4)
-    for epilogue in (1, 2):
-        info = fo._capi.kernel_info(algo, 8192, 8192, epilogue=epilogue, dtype=dtype)
-        assert info["resident"] == 256 and info["threads"] == 512 and info["lds_bytes"] <= 160 * 1024
-        assert 2 * ((info["vgprs"] + 7) // 8 * 8) + 64 <= 512, info
+    """The consumer kernels are built for one 64-register wavefront per SIMD beside the wavefronts
+    of a signalling GEMM workgroup (one per SIMD for the 256x256 tile, two for the smaller ones):
+    the GEMM's registers per SIMD (architectural + accumulation, allocated in eights) + 64 must fit
+    the 512 of a SIMD, or the overlapped path silently degrades into a serial one."""
+    for bm, bn, M, N in ((128, 256, 8192, 8192), (128, 256, 4224, 2048), (128, 128, 4224, 4224)):
+        algo = _algo(fo, bm, bn, swizzle=4)
+        for epilogue in (1, 2):
+            info = fo._capi.kernel_info(algo, M, N, epilogue=epilogue, dtype=dtype)
+            per_cu = info["resident"] // 256
+            assert info["resident"] == 256 * per_cu and per_cu * info["lds_bytes"] <= 160 * 1024
+            per_simd = per_cu * info["threads"] // 256
+            assert per_simd * ((info["vgprs"] + 7) // 8 * 8) + 64 <= 512, info
 
 
 def test_error_codes_on_gpu(fo):
