@@ -150,6 +150,26 @@ def test_signal_gemm_three_slot_shapes_walk_several_tiles(fo, oracle, dtype, K, 
     _signal_case(fo, oracle, dtype, bm, bn, M, N, K, cseg, W=W, swizzle=4, seed=11 + K)
 
 
+@pytest.mark.parametrize("dtype,bm,bn,K,cseg,W,monitor", [
+    (F16, 128, 256, 64, [400, 400], 0, False),         # one K step per tile: every step starts a tile, every epilogue is followed by loads
+    (F16, 128, 128, 128, [1] * 600 + [1000], 0, False),  # two K steps: the loader is always in the next tile; groups beyond the register table
+    (BF16, 256, 128, 200, [144, 256, 400], 0, False),  # three full K steps and a partial one (zeros from beyond the buffer range)
+    (F16, 128, 256, 192, [500, 300], 2, False),        # row-mapped stores
+    (F16, 128, 256, 72, [800], 0, True),               # monitor stamps, partial second K step
+    (BF16, 128, 128, 328, [800, 800], 4, False),       # row-mapped stores, five full K steps and a partial one
+])
+def test_signal_gemm_256_tile_walks_several_tiles(fo, oracle, dtype, bm, bn, K, cseg, W, monitor):
+    """The 256x256 workgroup tile (four wavefronts, operands straight into LDS through buffer loads, the
+    loader running two K steps ahead across tile boundaries).  400 tiles of 256x256 on 256 resident
+    workgroups: 144 workgroups compute a second tile, whose operands are requested during the first
+    tile's last steps, whose first meeting waits for the first tile's stores, and from whose first K
+    step the first tile's signal is sent."""
+    M, N = 6400, 4096
+    info = fo._capi.kernel_info(_algo(fo, bm, bn, swizzle=4), M, N, epilogue=2 if W else 1, dtype=dtype)
+    assert info["resident"] == 256 and info["threads"] == 256 and info["lds_bytes"] == 2 * 65536 + 4 * 16 * 136 * 2
+    _signal_case(fo, oracle, dtype, bm, bn, M, N, K, cseg, W=W, monitor=monitor, swizzle=4, seed=21 + K)
+
+
 @pytest.mark.parametrize("dtype", [F16, BF16])
 @pytest.mark.parametrize("bm,bn,M,N,K", [(128, 128, 256, 384, 8), (128, 128, 256, 384, 72),
                                          (128, 128, 384, 256, 200), (128, 128, 256, 256, 1376),

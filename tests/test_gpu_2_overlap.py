@@ -643,16 +643,17 @@ def test_overlap_with_a_partial_last_wave(fo, fused):
 
 
 @pytest.mark.parametrize("fused", [0, 1])
-@pytest.mark.parametrize("bm,bn,M,N", [(128, 256, 4224, 2048), (256, 128, 2048, 4224)])
-def test_overlap_on_three_slot_shapes(fo, fused, bm, bn, M, N):
-    """The overlapped call on the 128x256 / 256x128 workgroup tiles with more tiles (264) than resident
-    workgroups (256): the tiles of the second round are signalled from inside the K loop with operand
-    loads in flight, and the consumer on the other stream must still see every tile complete."""
-    K = 1096
+@pytest.mark.parametrize("bm,bn,M,N,K,cseg", [(128, 256, 4224, 2048, 1096, [128, 128, 8]),
+                                               (256, 128, 2048, 4224, 1096, [128, 128, 8]),
+                                               (128, 256, 6400, 4096, 136, [256, 256, 288])])
+def test_overlap_on_three_slot_shapes(fo, fused, bm, bn, M, N, K, cseg):
+    """The overlapped call with more workgroup tiles than resident workgroups: 264 tiles of 128x256 /
+    256x128 (rings of three slots) and 400 tiles of 256x256 on 256 workgroups.  The tiles of the
+    second round are signalled from inside the K loop with operand loads in flight, and the consumer
+    on the other stream must still see every tile complete."""
     algo = fo._capi.find_algo(bm, bn, swizzle=4)
     TM, TN = M // bm, N // bn
     T = TM * TN
-    cseg = [128, 128, 8]
     assert sum(cseg) == T and fo._capi.kernel_info(algo, M, N)["resident"] == 256
     g = torch.Generator(device="cuda").manual_seed(78)
     A = torch.randn(M, K, device="cuda", generator=g).half()
