@@ -23,7 +23,7 @@ PEAK_TFLOPS = 2516.6   # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the signal GEMM, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
 # profiles/gemm_c5_hbm_traffic.md (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 256 MiB copy).
-MEASURED_TRAFFIC_BYTES = {("c5", "f16"): 838479.1 * 1024 * 2.0 + 131136.0 * 1024}
+MEASURED_TRAFFIC_BYTES = {("c5", "f16"): 786630.0 * 1024 * 2.0 + 131100.0 * 1024}
 
 WORKLOADS = {
     # name: (M, N, K, BM, BN, dtype, group tiles, W, description)
@@ -259,7 +259,7 @@ def measure(args, workload, compact=False):
                    if (args.fused < 0 and 2.0 * M * N * K < 6.4e10)
                    else "one wait and one consumer launch per GEMM wave" if (args.fused == 0 or (args.fused < 0 and len(cseg) <= 16))
                    else "one"},
-        "roofline": {"bound": "mfma", "kernel": "fo_gemm_kernel (signal epilogue)",
+        "roofline": {"bound": "mfma", "kernel": "fo_gemm256_kernel (signal epilogue)",
                      "achieved": achieved, "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_TFLOPS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get((workload, dt)),
