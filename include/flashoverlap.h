@@ -71,10 +71,12 @@ int fo_workgroup_tiles(int algo, int M, int N, int32_t *tiles_per_workgroup, int
 int fo_gemm_wave_tiles(int dtype, int algo, int M, int N, int32_t *tiles);
 /* What the main launch of a problem occupies on the device (needs a GPU; no
  * counterpart in the reference): info = {resident workgroups, vector
- * registers per lane, LDS bytes per workgroup, threads per workgroup} of the
- * kernel with the given epilogue (0 plain, 1 signal, 2 scatter).  The consumer
- * kernels are built for one 64-register wavefront per SIMD beside two GEMM
- * wavefronts: that holds while the register count stays at or below 224. */
+ * registers per lane (architectural + accumulation), LDS bytes per workgroup,
+ * threads per workgroup} of the kernel with the given epilogue (0 plain,
+ * 1 signal, 2 scatter).  The consumer kernels are built for one 64-register
+ * wavefront per SIMD beside the GEMM's wavefronts (threads / 256 per SIMD and
+ * workgroup): that holds while GEMM wavefronts per SIMD x registers stays at or
+ * below 448. */
 int fo_gemm_kernel_info(int dtype, int algo, int M, int N, int epilogue, int32_t info[4]);
 
 /* ---- GEMM -------------------------------------------------------------
