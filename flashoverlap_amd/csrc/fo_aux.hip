@@ -623,7 +623,7 @@ int fo_fill_words(int32_t *words, int n, int value, fo_stream_t stream) {
 }
 
 int fo_consumer_reduce_with(int dtype, const void *src, void *acc, int64_t nelem, int W, int64_t seg_stride,
-                            void *own, int rank, bool stream_acc, fo_stream_t stream) {
+                            void *own, int rank, bool stream_acc, fo_stream_t stream, bool beside_gemm) {
     if (!src || !acc || nelem < 0 || W <= 0) return FO_ERR_ARG;
     if (own && (rank < 0 || rank >= W)) return FO_ERR_ARG;
     if (nelem == 0) return FO_OK;
@@ -637,12 +637,13 @@ int fo_consumer_reduce_with(int dtype, const void *src, void *acc, int64_t nelem
     }
     dim3 grid(consumer_grid(chunk16 * W, stream_acc)), block(CONSUMER_THREADS);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const int lds = beside_gemm ? kBesideGemmLds : 0;
     if (dtype == FO_F16)
-        hipLaunchKernelGGL(fo_consumer_kernel<fo_f16_tag>, grid, block, 0, s, (const fo_u32x4 *)src,
+        hipLaunchKernelGGL(fo_consumer_kernel<fo_f16_tag>, grid, block, lds, s, (const fo_u32x4 *)src,
                            (fo_u32x4 *)acc, chunk16, W, (long)(seg_stride / 8), (fo_u32x4 *)own, rank,
                            (int)stream_acc);
     else if (dtype == FO_BF16)
-        hipLaunchKernelGGL(fo_consumer_kernel<fo_bf16_tag>, grid, block, 0, s, (const fo_u32x4 *)src,
+        hipLaunchKernelGGL(fo_consumer_kernel<fo_bf16_tag>, grid, block, lds, s, (const fo_u32x4 *)src,
                            (fo_u32x4 *)acc, chunk16, W, (long)(seg_stride / 8), (fo_u32x4 *)own, rank,
                            (int)stream_acc);
     else
@@ -661,7 +662,7 @@ extern "C" int fo_consumer_reduce_rs_own(int dtype, const void *src, void *acc, 
 
 int fo_consumer_reduce_groups_with(int dtype, const void *src, void *acc, const int32_t *cseg_dev, int ngroups,
                                    int64_t max_group_tiles, int64_t tile_elems, int W, int64_t seg_stride,
-                                   void *own, int rank, bool stream_acc, fo_stream_t stream) {
+                                   void *own, int rank, bool stream_acc, fo_stream_t stream, bool beside_gemm) {
     if (!src || !acc || !cseg_dev || ngroups <= 0 || max_group_tiles <= 0 || tile_elems <= 0 || W < 2)
         return FO_ERR_ARG;
     if (own && (rank < 0 || rank >= W)) return FO_ERR_ARG;
@@ -674,12 +675,13 @@ int fo_consumer_reduce_groups_with(int dtype, const void *src, void *acc, const 
     if (per_group < 1) per_group = 1;
     dim3 grid(per_group, ngroups), block(CONSUMER_THREADS);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const int lds = beside_gemm ? kBesideGemmLds : 0;
     if (dtype == FO_F16)
-        hipLaunchKernelGGL(fo_consumer_groups_kernel<fo_f16_tag>, grid, block, 0, s, (const fo_u32x4 *)src,
+        hipLaunchKernelGGL(fo_consumer_groups_kernel<fo_f16_tag>, grid, block, lds, s, (const fo_u32x4 *)src,
                            (fo_u32x4 *)acc, cseg_dev, tile16, W, (long)(seg_stride / 8), (fo_u32x4 *)own, rank,
                            (int)stream_acc);
     else if (dtype == FO_BF16)
-        hipLaunchKernelGGL(fo_consumer_groups_kernel<fo_bf16_tag>, grid, block, 0, s, (const fo_u32x4 *)src,
+        hipLaunchKernelGGL(fo_consumer_groups_kernel<fo_bf16_tag>, grid, block, lds, s, (const fo_u32x4 *)src,
                            (fo_u32x4 *)acc, cseg_dev, tile16, W, (long)(seg_stride / 8), (fo_u32x4 *)own, rank,
                            (int)stream_acc);
     else

@@ -349,7 +349,8 @@ int allreduce_overlap(fo_overlap *h, int dtype, int M, int N, int K, const void 
                 if (rc) return rc;
             }
             if (acc) {  // the groups of a batch are one contiguous range
-                rc = fo_consumer_reduce_with(dtype, c + off, acc + off, n, 1, 0, nullptr, 0, stream_acc, cstream);
+                rc = fo_consumer_reduce_with(dtype, c + off, acc + off, n, 1, 0, nullptr, 0, stream_acc, cstream,
+                                             j < G && !same_stream);  // every batch but the last runs beside the GEMM
                 if (rc) return rc;
             }
             off += n;
@@ -446,14 +447,15 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
             for (int g = i; g < j; g++) most = cseg_host[g] > most ? cseg_host[g] : most;
             rc = fo_consumer_reduce_groups_with(dtype, c + off, acc + off / W, cseg_dev + i, j - i, most,
                                                 tile_elems, W, seg_stride, own_in_consumer ? d + off / W : nullptr,
-                                                h->rank, stream_acc, cstream);
+                                                h->rank, stream_acc, cstream, j < G && !same_stream);
             if (rc) return rc;
         }
         for (int g = i; g < j; g++) {
             const int64_t n = cseg_host[g] * tile_elems;
             if (!fused && acc && !(W > 1 && j - i > 1)) {
                 rc = fo_consumer_reduce_with(dtype, c + off, acc + off / W, n, W, seg_stride,
-                                             own_in_consumer ? d + off / W : nullptr, h->rank, stream_acc, cstream);
+                                             own_in_consumer ? d + off / W : nullptr, h->rank, stream_acc, cstream,
+                                             j < G && !same_stream);
                 if (rc) return rc;
             }
             if (d && !own_in_consumer)
