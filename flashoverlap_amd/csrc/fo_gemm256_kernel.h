@@ -280,6 +280,22 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
             }
         }
     };
+    // Storage slots of a macro tile's reorder tiles (scalar loads).  They are requested one tile ahead (in front of
+    // the pipeline fill for the first tile, in front of the previous tile's epilogue otherwise) and awaited at the
+    // tile's start: the round trip to memory then costs nothing, and no scalar load is pending at the K loop's head,
+    // where it would turn every wait for LDS data into a wait for everything (scalar loads return out of order).
+    int rs_next[kMaxSub] = {0, 0, 0, 0};
+    auto request_slots = [&](int t) {
+        if (MODE != MODE_PLAIN) {
+            int tm_, tn_;
+            fo_unit_to_tile(t, p.first, p.sub_m, p.sub_n, p.grid_m, p.grid_n, p.panel, p.xcd_remap, &tm_, &tn_);
+            tm_ = __builtin_amdgcn_readfirstlane(tm_);
+            tn_ = __builtin_amdgcn_readfirstlane(tn_);
+#pragma unroll
+            for (int s = 0; s < kMaxSub; s++)
+                if (s < nsub) rs_next[s] = RAc[(tm_ * (MT / p.BM) + s / sub_n) * p.TN + tn_ * sub_n + s % sub_n];
+        }
+    };
     int prev_rs[kMaxSub] = {0, 0, 0, 0};  // slots and groups of the tile whose signal is still owed
     int prev_gs[kMaxSub] = {0, 0, 0, 0};
     int owed = 0;          // PUB meetings until that signal may be sent
@@ -294,6 +310,7 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
     };
 
     // ---- pipeline fill: stage 0 -> slot 0, stage 1 -> slot 1; the loader then stands at stage 1
+    request_slots(blockIdx.x);
     set_loader_tile();
 #pragma unroll
     for (int c = 0; c < 16; c++) load_chunk(c, 0);
@@ -315,15 +332,13 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
         fo_unit_to_tile(tile, p.first, p.sub_m, p.sub_n, p.grid_m, p.grid_n, p.panel, p.xcd_remap, &pm, &pn);
         pm = __builtin_amdgcn_readfirstlane(pm);
         pn = __builtin_amdgcn_readfirstlane(pn);
-        int rs[kMaxSub] = {0, 0, 0, 0};  // storage slots of this macro tile's reorder tiles (scalar loads)
+        int rs[kMaxSub] = {0, 0, 0, 0};  // storage slots of this macro tile's reorder tiles
         if (MODE != MODE_PLAIN) {
 #pragma unroll
-            for (int s = 0; s < kMaxSub; s++)
-                if (s < nsub) rs[s] = RAc[(pm * (MT / p.BM) + s / sub_n) * p.TN + pn * sub_n + s % sub_n];
-            // The scalar loads complete here: one still pending at the K loop's head would turn every wait for
-            // LDS data inside the loop into a wait for everything (scalar loads return out of order).
-#pragma unroll
-            for (int s = 0; s < kMaxSub; s++) asm volatile("" : "+s"(rs[s]));
+            for (int s = 0; s < kMaxSub; s++) {
+                rs[s] = rs_next[s];
+                asm volatile("" : "+s"(rs[s]));  // the scalar loads complete here
+            }
         }
 #pragma unroll
         for (int i = 0; i < F; i++)
@@ -428,6 +443,7 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
         fo_mfma_fence();
         const int next = tile + gridDim.x;
         const bool has_next = next < ntiles;
+        if (has_next) request_slots(next);
 
         // ---- epilogue.  A wavefront's 128x128 block lies inside one reorder tile (BM and BN are multiples of
         // 128), so slot and base address are scalars.  The lane id is laundered so that this addressing is
