@@ -9,6 +9,10 @@
 // src/overlap/gemm_signal.cu:15-97, src/overlap/gemm_scatter.cu:15-98; epilogue
 // semantics src/overlap/gemm_with_signal.h:236-256, :291-361).
 //
+// This template serves the 128x128, 128x256 and 256x128 workgroup tiles; the
+// 256x256 tile has a kernel of its own (fo_gemm256_kernel.h), which shares the
+// arguments, the raster and the helpers defined here.
+//
 // The kernel is persistent: the launch holds at most as many workgroups as the
 // chip keeps resident, and workgroup w computes macro tiles w, w + grid,
 // w + 2 grid, ... of the raster.  A workgroup of WM x WN wavefronts computes an
