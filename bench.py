@@ -48,6 +48,8 @@ def measure(args, workload, compact=False):
     algo = fo._capi.find_algo(BM, BN, swizzle=args.swizzle)
     TM, TN = M // BM, N // BN
     T = TM * TN
+    if args.comm_cus and not compact and not args.group_tiles:
+        gtiles = fo._capi.wave_tiles(algo, M, N)  # one group per GEMM wave, whatever the CU limit makes of a wave
     if workload == "c3" and (compact or not args.group_tiles):
         # wave-group sizes chosen by the predictive search (tune/search.py:442-502) from a measured
         # GEMM duration and the consumer's measured bandwidth curve
@@ -138,7 +140,54 @@ def measure(args, workload, compact=False):
         wall = (time.perf_counter() - t0) * 1e3 / steps
         return e0.elapsed_time(e1) / steps, wall
 
+    # Bring the part to its sustained clocks first: for the first few dozen launches after idle
+    # the same GEMM runs up to 30 % slower, which would otherwise fall on whatever is timed first.
+    def settle(fn, seconds=0.5):
+        t_end = time.perf_counter() + seconds
+        while time.perf_counter() < t_end:
+            for _ in range(20):
+                fn()
+            torch.cuda.synchronize()
+
     K_, W_ = (max(5, args.steps // 2), max(3, args.warmup // 2)) if compact else (args.steps, args.warmup)
+    if args.steps_only and not compact and args.comm_cus:
+        # CU-masked streams: the consumer's stream may use comm_cus CUs (the mask's low bits), the GEMM's
+        # all of them or, with --gemm-cus-disjoint, the others (the library was told to plan for that
+        # many in main()).  The call that takes both streams from the caller is the one without a handle.
+        import ctypes
+        if W:
+            raise SystemExit("--comm-cus: all-reduce workloads only")
+        hip = ctypes.CDLL("libamdhip64.so")
+        cus = torch.cuda.get_device_properties(0).multi_processor_count
+        nw = (cus + 31) // 32
+
+        def masked_stream(bits):
+            words = (ctypes.c_uint32 * nw)(*[(bits >> (32 * i)) & 0xFFFFFFFF for i in range(nw)])
+            s = ctypes.c_void_p()
+            rc = hip.hipExtStreamCreateWithCUMask(ctypes.byref(s), nw, words)
+            if rc:
+                raise SystemExit(f"hipExtStreamCreateWithCUMask: error {rc}")
+            return torch.cuda.ExternalStream(s.value)
+
+        comm_bits = (1 << args.comm_cus) - 1
+        comm_s = masked_stream(comm_bits)
+        gemm_s = masked_stream(((1 << cus) - 1) & ~comm_bits) if args.gemm_cus_disjoint else torch.cuda.Stream()
+        torch.cuda.synchronize()
+
+        def step_masked():
+            ops.gemm_allreduce_overlap_static(A, B, Cp, ACC, RA, 1, cs_cpu, cs_gpu, algo, fused=args.fused,
+                                              gemm_stream=gemm_s, comm_stream=comm_s)
+            norm()
+
+        with torch.cuda.stream(gemm_s):
+            settle(gemm_alone)
+            ms_g, _ = timed(gemm_alone, K_, W_)
+            ms, _ = timed(step_masked, K_, W_)
+        print(json.dumps({"steps_only": True, "steps": K_, "warmup": W_, "comm_cus": args.comm_cus,
+                          "gemm_cus": cus - args.comm_cus if args.gemm_cus_disjoint else cus,
+                          "wave_tiles": fo._capi.wave_tiles(algo, M, N), "cseg": cseg,
+                          "gemm_alone_ms": ms_g, "ms_per_step": ms}))
+        return
     if args.steps_only and not compact:
         ms, _ = timed(step_overlapped, K_, W_)
         print(json.dumps({"steps_only": True, "steps": K_, "warmup": W_, "ms_per_step": ms}))
@@ -150,15 +199,6 @@ def measure(args, workload, compact=False):
         torch.cuda.synchronize()
         print(json.dumps({"kernels_only": True, "steps": K_, "warmup": W_}))
         return
-    # Bring the part to its sustained clocks first: for the first few dozen launches after idle
-    # the same GEMM runs up to 30 % slower, which would otherwise fall on whatever is timed first.
-    def settle(fn, seconds=0.5):
-        t_end = time.perf_counter() + seconds
-        while time.perf_counter() < t_end:
-            for _ in range(20):
-                fn()
-            torch.cuda.synchronize()
-
     settle(step_serial, 0.25 if compact else 0.5)
     ms_step, wall_step = timed(step_overlapped, K_, W_)
     ms_serial, _ = timed(step_serial, K_, W_)
@@ -308,6 +348,11 @@ def main():
     ap.add_argument("--steps-only", action="store_true",
                     help="enqueue warmup + steps overlapped steps and exit: for a kernel-trace timeline of the "
                          "steady state")
+    ap.add_argument("--comm-cus", type=int, default=0,
+                    help="with --steps-only: put the consumer on a stream masked to this many CUs (a multiple of 8)")
+    ap.add_argument("--gemm-cus-disjoint", action="store_true",
+                    help="with --comm-cus: put the GEMM on a stream masked to the other CUs and let the library "
+                         "plan its launches for that many (fo_gemm_set_cu_limit)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a 256 MiB device-to-device copy five times (reference point for "
                          "scaling the FETCH_SIZE / WRITE_SIZE counters) and exit")
@@ -323,6 +368,11 @@ def main():
     from flashoverlap_amd import ops
 
     torch.cuda.set_device(0)
+    if args.comm_cus:
+        if not args.steps_only or args.comm_cus % 8 or args.comm_cus <= 0:
+            raise SystemExit("--comm-cus wants --steps-only and a positive multiple of 8")
+        if args.gemm_cus_disjoint:
+            fo._capi.set_gemm_cu_limit(torch.cuda.get_device_properties(0).multi_processor_count - args.comm_cus)
     if args.copy_calibration:
         src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
         dst = torch.empty_like(src)

@@ -60,6 +60,7 @@ SIGNATURES = {
                                               vp, c_int, c_int, c_int, vp, vp, c_int, c_int, c_int]),
     "fo_overlap_gemm_allreduce_serial": (c_int, [vp, c_int, c_int, c_int, c_int, vp, vp, vp, c_int]),
     "fo_overlap_seg_allreduce": (c_int, [vp, c_int, vp, c_i64, vp, c_int, c_int]),
+    "fo_gemm_set_cu_limit": (c_int, [c_int]),
     "fo_gemm_allreduce_overlap_static": (c_int, [c_int, c_int, c_int, c_int, vp, vp, vp, vp, vp, c_int, c_int, c_int,
                                                  vp, vp, c_int, c_int, c_int, vp, vp]),
 }
@@ -129,6 +130,12 @@ def schedule_order(algo, M, N):
     buf = (ctypes.c_int32 * T)()
     check(lib().fo_schedule_order(int(algo), M, N, buf), "fo_schedule_order")
     return list(buf)
+
+
+def set_gemm_cu_limit(n):
+    """The GEMM launches count on n CUs from here on (0: on all); the schedule order, wave_tiles and
+    kernel_info answer for that number, so take them again afterwards."""
+    check(lib().fo_gemm_set_cu_limit(int(n)), "fo_gemm_set_cu_limit")
 
 
 def wave_tiles(algo, M, N, dtype=F16):

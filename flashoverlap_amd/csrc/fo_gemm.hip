@@ -124,25 +124,38 @@ int run_gemm(int mode, int dtype, int M, int N, int K, int rLDN, const int32_t *
 // this number.  Without a usable device (host-only callers asking for the schedule order)
 // the answer is MI355X's: 256 CUs, one workgroup each.
 int fo_main_tile_resident() {
+    const int limit = gemm_cu_limit().load(std::memory_order_relaxed);
+    const int no_device = limit > 0 && limit < 256 ? limit / 8 * 8 : 256;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) {
         (void)hipGetLastError();
-        return 256;
+        return no_device;
     }
-    static std::atomic<int> cached[kMaxDevices];  // asked on every launch: answered from here after the first
+    // Asked on every launch: answered from here after the first.  An entry holds the CU limit it was
+    // computed under (plus one, in the upper half) and the answer.
+    static std::atomic<int> cached[kMaxDevices];
     if (dev >= 0 && dev < kMaxDevices) {
         const int c = cached[dev].load(std::memory_order_relaxed);
-        if (c > 0) return c;
+        if ((c >> 16) == limit + 1) return c & 0xFFFF;
     }
     GemmArgs a = {};
     a.count = 1 << 30;
     int info[5] = {0, 0, 0, 0, 0};
-    if (launch_dtype<MODE_SIGNAL>(FO_F16, a, 256, 256, nullptr, info) != FO_OK || info[4] <= 0) {
+    if (launch_dtype<MODE_SIGNAL>(FO_F16, a, 256, 256, nullptr, info) != FO_OK || info[4] <= 0 || info[4] > 0xFFFF) {
         (void)hipGetLastError();
-        return 256;
+        return no_device;
     }
-    if (dev >= 0 && dev < kMaxDevices) cached[dev].store(info[4], std::memory_order_relaxed);
+    if (dev >= 0 && dev < kMaxDevices) cached[dev].store((limit + 1) << 16 | info[4], std::memory_order_relaxed);
     return info[4];
+}
+
+// The GEMM launches count on n CUs from here on (n <= 0: on all).  Process-wide, read at every launch;
+// the caller changes it only while no schedule order taken under the old value is still in use.
+extern "C" int fo_gemm_set_cu_limit(int n) {
+    if (n > 0 && n < 8) return FO_ERR_ARG;  // the raster wants a workgroup count that is a multiple of the 8 XCDs
+    if (n > 0x7FFE) return FO_ERR_ARG;
+    gemm_cu_limit().store(n > 0 ? n : 0, std::memory_order_relaxed);
+    return FO_OK;
 }
 
 // The reordered (optionally row-mapped) store of the signalling GEMMs without

@@ -2,6 +2,7 @@
 // kernel instantiations (fo_gemm.hip, fo_gemm256_inst.hip).
 #pragma once
 
+#include <atomic>
 #include <mutex>
 
 #include "fo_gemm_kernel.h"
@@ -9,6 +10,15 @@
 namespace fo_gemm_dev {
 
 constexpr int kMaxDevices = 64;
+
+// CUs that the GEMM launches may count on (0: all of the device's).  A caller that keeps CUs for other
+// kernels, e.g. with CU-masked streams, says so through fo_gemm_set_cu_limit; the persistent launches
+// and the raster (with it the schedule order handed out as the hint) then assume that many CUs, as the
+// reference's tuner assumes sm_count - 2 (tune/search.py:404-407).
+inline std::atomic<int> &gemm_cu_limit() {
+    static std::atomic<int> limit{0};
+    return limit;
+}
 
 // One compiled shape of the kernel template.  The launch is persistent: as many
 // workgroups as the device keeps resident at once (or fewer, if the problem has
@@ -22,16 +32,16 @@ inline int launch_kernel(const GemmArgs &a, hipStream_t stream, int *resident_ou
     auto kern = KERN;
     constexpr int smem = SMEM;
     constexpr int threads = THREADS;
-    // Resident workgroups of this instantiation per device; the LDS attribute is set once per device too.
+    // CUs of each device and workgroups of this instantiation per CU; the LDS attribute is set once per device too.
     static std::mutex mu;
-    static int resident_of[kMaxDevices];
+    static int cus_of[kMaxDevices], per_cu_of[kMaxDevices];
     int dev = 0;
     FO_HIP_CHECK(hipGetDevice(&dev));
     if (dev < 0 || dev >= kMaxDevices) return FO_ERR_STATE;
     int resident;
     {
         std::lock_guard<std::mutex> lock(mu);
-        if (!resident_of[dev]) {
+        if (!per_cu_of[dev]) {
             FO_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, smem));
             int cus = 0, per_cu = 0;
@@ -39,11 +49,14 @@ inline int launch_kernel(const GemmArgs &a, hipStream_t stream, int *resident_ou
             FO_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(kern),
                                                                       threads, smem));
             if (cus <= 0 || per_cu <= 0) return FO_ERR_STATE;
-            // a multiple of 8 keeps "workgroup id mod 8 = XCD" true for every tile of the walk
-            int r = (cus * per_cu) / 8 * 8;
-            resident_of[dev] = r > 0 ? r : cus * per_cu;
+            cus_of[dev] = cus;
+            per_cu_of[dev] = per_cu;
         }
-        resident = resident_of[dev];
+        const int limit = gemm_cu_limit().load(std::memory_order_relaxed);
+        const int cus = limit > 0 && limit < cus_of[dev] ? limit : cus_of[dev];
+        // a multiple of 8 keeps "workgroup id mod 8 = XCD" true for every tile of the walk
+        const int r = (cus * per_cu_of[dev]) / 8 * 8;
+        resident = r > 0 ? r : cus * per_cu_of[dev];
     }
     // The raster (and with it the schedule order handed to the caller as the hint) was laid out for
     // expect_resident workgroups; a launch that would hold another number walks the tiles differently.

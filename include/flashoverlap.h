@@ -78,6 +78,16 @@ int fo_gemm_wave_tiles(int dtype, int algo, int M, int N, int32_t *tiles);
  * workgroup): that holds while GEMM wavefronts per SIMD x registers stays at or
  * below 448. */
 int fo_gemm_kernel_info(int dtype, int algo, int M, int N, int epilogue, int32_t info[4]);
+/* The GEMM launches count on n CUs from this call on (n <= 0: on all of the
+ * device's; 0 < n < 8 is FO_ERR_ARG): the persistent launches hold
+ * n x workgroups-per-CU workgroups (rounded down to a multiple of 8), and
+ * fo_schedule_order, fo_gemm_wave_tiles and fo_gemm_kernel_info answer for that
+ * number.  For a caller that keeps CUs for other kernels, e.g. by putting the
+ * consumer on a CU-masked stream and the GEMM on a stream masked to the rest.
+ * Process-wide; take the schedule order (and the RA built from it) again after
+ * changing it.  The reference assumes sm_count - 2 SMs for the GEMM in the same
+ * places (tune/search.py:404-407, :459-464, test/test.py:330). */
+int fo_gemm_set_cu_limit(int n);
 
 /* ---- GEMM -------------------------------------------------------------
  * C[M,N] = A[M,K] . B[N,K]^T, 16-bit in/out, fp32 accumulate.

@@ -170,6 +170,26 @@ def test_signal_gemm_256_tile_walks_several_tiles(fo, oracle, dtype, bm, bn, K, 
     _signal_case(fo, oracle, dtype, bm, bn, M, N, K, cseg, W=W, monitor=monitor, swizzle=4, seed=21 + K)
 
 
+def test_signal_gemm_under_a_cu_limit(fo, oracle):
+    """fo_gemm_set_cu_limit (the reference plans for sm_count - 2, tune/search.py:404-407): with 96 CUs
+    the persistent launch holds 96 workgroups, a wave is 96 x 2 reorder tiles of 128x256, and the 400
+    tiles of 256x256 are four full waves and a tail of 16 that a second launch walks in the Algo's own
+    tile; counters, reordered stores and values as ever."""
+    M, N, bm, bn = 6400, 4096, 128, 256
+    algo = _algo(fo, bm, bn, swizzle=4)
+    try:
+        fo._capi.set_gemm_cu_limit(96)
+        info = fo._capi.kernel_info(algo, M, N, epilogue=1, dtype=F16)
+        assert info["resident"] == 96
+        assert fo._capi.wave_tiles(algo, M, N) == 192
+        _signal_case(fo, oracle, F16, bm, bn, M, N, 136, [500, 144, 156], swizzle=4, seed=77)
+        _signal_case(fo, oracle, BF16, 128, 128, M, N, 64, [1600], swizzle=4, seed=78, monitor=True)
+    finally:
+        fo._capi.set_gemm_cu_limit(0)
+    assert fo._capi.kernel_info(algo, M, N, epilogue=1, dtype=F16)["resident"] == 256
+    assert fo._capi.wave_tiles(algo, M, N) == 512
+
+
 @pytest.mark.parametrize("dtype", [F16, BF16])
 @pytest.mark.parametrize("bm,bn,M,N,K", [(128, 128, 256, 384, 8), (128, 128, 256, 384, 72),
                                          (128, 128, 384, 256, 200), (128, 128, 256, 256, 1376),

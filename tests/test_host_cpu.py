@@ -82,6 +82,33 @@ def test_schedule_order_with_a_partial_last_wave():
     assert sorted(order2) == list(range((M // 256) * (N // 128)))
 
 
+def test_cu_limit_is_accepted_and_keeps_the_hint_a_permutation():
+    """fo_gemm_set_cu_limit (the reference's sm_count - 2, tune/search.py:404-407): 1024 workgroup tiles
+    are four full waves on 256 CUs, and four waves of 248 plus a tail of 32 on 248 CUs.  The tail is
+    walked in the Algo's own 128x128 tile, position by position, so the hint stays the raster's order
+    of 256x256 blocks either way; what changes with the limit (wave sizes, resident workgroups) needs
+    the GPU and is tested there."""
+    L = _capi.lib()
+    assert L.fo_gemm_set_cu_limit(4) == -1      # fewer than the 8 XCDs
+    algo = _capi.find_algo(128, 128, swizzle=4)
+    M = N = 8192
+    full = _capi.schedule_order(algo, M, N)
+    try:
+        _capi.set_gemm_cu_limit(248)
+        cut = _capi.schedule_order(algo, M, N)
+        _capi.set_gemm_cu_limit(512)            # more than the device has: all of them
+        assert _capi.schedule_order(algo, M, N) == full
+    finally:
+        _capi.set_gemm_cu_limit(0)
+    assert _capi.schedule_order(algo, M, N) == full
+    T = (M // 128) * (N // 128)
+    tn = N // 128
+    assert sorted(cut) == list(range(T))
+    for i in range(0, T, 4):
+        a, b, c, d = cut[i:i + 4]
+        assert b == a + 1 and c == a + tn and d == c + 1
+
+
 def test_argument_validation_without_gpu():
     L = _capi.lib()
     null = ctypes.c_void_p()
