@@ -15,6 +15,7 @@ using namespace fo_gemm_dev;
 
 int fo_gemm_dev::fo_gemm256_launch(int dtype, int mode, const GemmArgs &a, hipStream_t stream, int *resident_out,
                                    int expect_resident) {
+    if (a.lda != a.ldb) return FO_ERR_ARG;  // the kernel addresses both operands with one leading dimension
     const int key = (dtype == FO_BF16 ? 3 : 0) + mode;
     switch (key) {
         case 0: return fo_gemm256_launch_0_0(a, stream, resident_out, expect_resident);

@@ -143,23 +143,22 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
     const int lrow = lane >> 3;
     const int lchunk = (lane & 7) ^ (((wave * 8 + lrow) >> 1) & 7);
     const unsigned a_off = (unsigned)((wave * 8 + lrow) * p.lda * 2 + lchunk * 16);
-    const unsigned b_off = (unsigned)((wave * 8 + lrow) * p.ldb * 2 + lchunk * 16);
     const bool tail_out = (KT - 1) * BK + lchunk * 8 >= p.K;  // this lane's chunk of the last K step lies beyond K
     const unsigned a_off_t = tail_out ? 0x80000000u : a_off;  // beyond every descriptor's range
-    const unsigned b_off_t = tail_out ? 0x80000000u : b_off;
     // The descriptors point at the stage's first column of the tile's first row and cover exactly the
     // tile's rows from there (the host checks that this fits 31 bits).
-    const unsigned a_span = (unsigned)((255 * p.lda + p.K) * 2), b_span = (unsigned)((255 * p.ldb + p.K) * 2);
-    unsigned soff_a[8], soff_b[8];  // row-block offsets of the eight loads per operand
+    const unsigned a_span = (unsigned)((255 * p.lda + p.K) * 2);
+    // A and B have one leading dimension (the launcher checks it), so the lane offsets, the span and the
+    // row-block offsets of the eight loads per operand serve both.
+    unsigned soff_a[8];
 #pragma unroll
     for (int c = 0; c < 8; c++) {
         soff_a[c] = __builtin_amdgcn_readfirstlane((unsigned)(c * 32 * p.lda * 2));
-        soff_b[c] = __builtin_amdgcn_readfirstlane((unsigned)(c * 32 * p.ldb * 2));
     }
 
     // Loader state: the stage being requested (it runs two K steps ahead of the MFMAs, across tiles).
     int ld_tile = blockIdx.x, ld_kt = 0;
-    unsigned a_cur = (ktail && KT == 1) ? a_off_t : a_off, b_cur = (ktail && KT == 1) ? b_off_t : b_off;
+    unsigned a_cur = (ktail && KT == 1) ? a_off_t : a_off;  // this stage's lane offsets, A and B alike
     fo_srd_t ra, rb;
     auto make_srd = [&](const void *base, unsigned records) {
         const uint64_t b = (uint64_t)(uintptr_t)base;
@@ -177,7 +176,7 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
             pm_ = __builtin_amdgcn_readfirstlane(pm_);
             pn_ = __builtin_amdgcn_readfirstlane(pn_);
             ra = make_srd(p.A + (size_t)pm_ * MT * p.lda, a_span);
-            rb = make_srd(p.B + (size_t)pn_ * MT * p.ldb, b_span);
+            rb = make_srd(p.B + (size_t)pn_ * MT * p.lda, a_span);
         } else {
             ra = make_srd(p.A, 0);  // behind the last tile: every load is out of range, nothing is fetched
             rb = make_srd(p.B, 0);
@@ -202,7 +201,6 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
         if (ktail) {
             const bool t = ld_kt == KT - 1;
             a_cur = t ? a_off_t : a_off;
-            b_cur = t ? b_off_t : b_off;
         }
     };
     // load c of the loader's stage into the slot at byte offset `slot` (pipeline fill)
@@ -210,15 +208,14 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
         if (c < 8)
             dma_buf16(ra, a_cur, soff_a[c & 7], (wa0 ^ slot) + c * CHUNK_B);
         else
-            dma_buf16(rb, b_cur, soff_b[c & 7], (wa0 ^ slot) + c * CHUNK_B);
+            dma_buf16(rb, a_cur, soff_a[c & 7], (wa0 ^ slot) + c * CHUNK_B);
     };
     // the same riding on an MFMA (K loop)
     auto mfma_load_chunk = [&](fo_u32x4 x, fo_u32x4 y, fo_float4v &cc, int c, unsigned lds_base) {
         switch (c) {
 #define FO_CASE(C_)                                                                                           \
     case C_:                                                                                                  \
-        X::template go_load<C_ * CHUNK_B>(x, y, cc, lds_base, C_ < 8 ? ra : rb, C_ < 8 ? a_cur : b_cur,       \
-                                          C_ < 8 ? soff_a[C_ & 7] : soff_b[C_ & 7]);                          \
+        X::template go_load<C_ * CHUNK_B>(x, y, cc, lds_base, C_ < 8 ? ra : rb, a_cur, soff_a[C_ & 7]);       \
         break;
             FO_CASE(0) FO_CASE(1) FO_CASE(2) FO_CASE(3) FO_CASE(4) FO_CASE(5) FO_CASE(6) FO_CASE(7)
             FO_CASE(8) FO_CASE(9) FO_CASE(10) FO_CASE(11) FO_CASE(12) FO_CASE(13) FO_CASE(14) FO_CASE(15)
