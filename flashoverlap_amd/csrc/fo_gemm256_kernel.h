@@ -261,14 +261,24 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
     // Wavefront 0 announces the reorder tiles at slots rs[] with groups gs[].  Callers guarantee that every
     // wavefront's write-through stores of those tiles are acknowledged (vmcnt) and that a workgroup barrier
     // lies between that wait and this call, so the atomic itself is relaxed.
+    // Reorder tiles of one group are counted with one atomic: all resident workgroups finish a tile at about the
+    // same time and bump the same few counters, and atomics on one address complete one after the other, some 25 ns
+    // apart (512 tiles of 256x256 in 128x128 reorder tiles, 8 groups: 7 us per launch with one atomic per tile).
     auto announce = [&](const int (&rs)[kMaxSub], const int (&gs)[kMaxSub]) {
 #pragma unroll
         for (int s = 0; s < kMaxSub; s++) {
             if (s < nsub) {
                 const int r = rs[s];
                 const int g = gs[s];
+                int count = 1;       // tiles s, s+1, ... of this group
+                bool first = true;   // no earlier tile of this group
+#pragma unroll
+                for (int q = 0; q < kMaxSub; q++) {
+                    if (q < s && gs[q] == g) first = false;
+                    if (q > s && q < nsub && gs[q] == g) count++;
+                }
                 if (lane == 0) {
-                    __hip_atomic_fetch_add(p.MM + g, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (first) __hip_atomic_fetch_add(p.MM + g, count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     if (p.monitor) {
                         int o = __hip_atomic_fetch_add(p.MM + (p.TN - 1), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                         __hip_atomic_store(p.MM + p.TN + r, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -336,6 +346,17 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
                 rs[s] = rs_next[s];
                 asm volatile("" : "+s"(rs[s]));  // the scalar loads complete here
             }
+        }
+        // Scatter: the row map entries of the wavefront's 128 rows, two per lane (lane l: rows l and 64 + l), are
+        // requested here and rest in two registers through the K loop; the epilogue hands them to the lanes that
+        // store each row.  Requested in the epilogue they cost every tile a round trip to memory with nothing to hide it.
+        int32_t re_lo = 0, re_hi = 0;
+        if (MODE == MODE_SCATTER) {
+            const int s = ((wm * 128) / p.BM) * sub_n + (wn * 128) / p.BN;
+            const int r = s == 0 ? rs[0] : s == 1 ? rs[1] : s == 2 ? rs[2] : rs[3];
+            const long trow = (long)(r / p.rLDN) * p.BM + (wm * 128) % p.BM;
+            re_lo = p.RE[trow + lane];
+            re_hi = p.RE[trow + 64 + lane];
         }
 #pragma unroll
         for (int i = 0; i < F; i++)
@@ -462,15 +483,6 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
             const long tcol = MODE == MODE_PLAIN ? (long)pn * MT + wn * 128 : (long)(r % p.rLDN) * p.BN + col0;
             char *cbase = reinterpret_cast<char *>(p.C) + (trow * ldp + tcol) * 2;  // wave-uniform
             const unsigned lane_off = (unsigned)(srow * ldp + scol * 8) * 2;
-            // scatter: the row map entries of all rows this lane will store, fetched in one batch
-            int32_t dest_row[MODE == MODE_SCATTER ? NST : 1];
-            if (MODE == MODE_SCATTER) {
-#pragma unroll
-                for (int i = 0; i < F; i++)
-#pragma unroll
-                    for (int ps = 0; ps < 16 / RPP; ps++)
-                        dest_row[i * (16 / RPP) + ps] = p.RE[trow + i * 16 + ps * RPP + srow];
-            }
 #pragma unroll
             for (int i = 0; i < F; i++) {  // 16 output rows = one row of accumulator blocks
                 __builtin_amdgcn_sched_barrier(0);
@@ -496,7 +508,9 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
                     const int row = ps * RPP + srow;
                     fo_u32x4 v = *reinterpret_cast<const fo_u32x4 *>(strip + row * PITCH + scol * 8);
                     if (MODE == MODE_SCATTER) {
-                        const long prow = dest_row[i * (16 / RPP) + ps];
+                        // row i * 16 + ps * RPP + srow of the block: its entry sits in that lane of re_lo / re_hi
+                        const long prow = __builtin_amdgcn_ds_bpermute(((i * 16 + ps * RPP) % 64 + srow) * 4,
+                                                                       i * 16 + ps * RPP < 64 ? re_lo : re_hi);
                         store16_write_through(p.C + (size_t)prow * ldp + tcol + scol * 8, v);
                     } else {
                         char *sb = cbase + (size_t)(i * 16 + ps * RPP) * ldp * 2;
