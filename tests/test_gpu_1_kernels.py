@@ -380,6 +380,24 @@ def test_streaming_forms_give_the_same_bits(fo, dtype):
     fo.ops.rmsnorm(X[:bm], Yps, Wt, eps=1e-6)
     torch.cuda.synchronize()
     assert torch.equal(Yp[:bm], Yps)
+    # Rows from the middle and the end of a streaming-size matrix whose row count is no multiple of the
+    # workgroup's four rows (the last workgroup's spare wavefronts lie beyond it) against runs on those
+    # rows alone, which take the cacheable form.
+    bs2 = M - 3
+    Yq = torch.full((M, N), float("nan"), device="cuda", dtype=td)
+    fo.ops.rmsnorm(X[:bs2], Yq[:bs2], Wt, eps=1e-6)
+    for lo, hi in ((bs2 - 69, bs2), (4001, 4090)):
+        Yqs = torch.empty(hi - lo, N, device="cuda", dtype=td)
+        fo.ops.rmsnorm(X[lo:hi], Yqs, Wt, eps=1e-6)
+        torch.cuda.synchronize()
+        assert torch.equal(Yq[lo:hi], Yqs)
+        assert torch.equal(Yp[lo:hi], Yqs)
+    assert torch.isnan(Yq[bs2:]).all()                       # nothing written beyond the last row
+    lo = 37 * bm                                             # a tile row from the middle, reordered form
+    Yrs = torch.empty(bm, N, device="cuda", dtype=td)
+    fo.ops.reorder_rmsnorm(X[lo:lo + bm], Yrs, Wt, bm, bn, 1, (RA[37:38] - 37 * TN).contiguous(), eps=1e-6)
+    torch.cuda.synchronize()
+    assert torch.equal(Y[lo:lo + bm], Yrs)
 
 
 @pytest.mark.parametrize("dtype", [F16, BF16])
