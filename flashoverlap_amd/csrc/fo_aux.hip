@@ -635,7 +635,8 @@ int fo_consumer_reduce_with(int dtype, const void *src, void *acc, int64_t nelem
                                     static_cast<hipStream_t>(stream)));
         own = nullptr;
     }
-    dim3 grid(consumer_grid(chunk16 * W, stream_acc)), block(CONSUMER_THREADS);
+    dim3 grid(consumer_grid(chunk16 * W, stream_acc));
+    dim3 block(beside_gemm && stream_acc && W == 1 ? kBesideGemmThreads : CONSUMER_THREADS);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int lds = beside_gemm ? kBesideGemmLds : 0;
     if (dtype == FO_F16)

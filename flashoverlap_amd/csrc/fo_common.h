@@ -118,6 +118,12 @@ inline bool fo_streams(int64_t bytes) { return bytes > kStreamAboveBytes; }
 // up to eight: the consumer's loads share each CU's load path with the GEMM's
 // operand stream (8192^3: overlapped step 0.842 instead of 0.847 ms).
 constexpr int kBesideGemmLds = 12288;
+// A streaming all-reduce consumer beside the GEMM also runs with one wavefront per workgroup instead of
+// four, i.e. on one of the CU's four SIMDs: same grid, a quarter of the lanes, each moving four times as
+// much.  Alone it would be slower; beside the GEMM it takes less from it (8192^3: overlapped step 0.846
+// against 0.855 ms, 8192x8192x3584: 0.410 against 0.424, alternating runs on one box).  The
+// reduce-scatter layout and cacheable accumulators lose that way and keep four wavefronts.
+constexpr int kBesideGemmThreads = 64;
 int fo_consumer_reduce_with(int dtype, const void *src, void *acc, int64_t nelem, int W, int64_t seg_stride,
                             void *own, int rank, bool stream_acc, fo_stream_t stream, bool beside_gemm = false);
 int fo_consumer_reduce_groups_with(int dtype, const void *src, void *acc, const int32_t *cseg_dev, int ngroups,
