@@ -183,6 +183,7 @@ def measure(args, workload, compact=False):
             settle(gemm_alone)
             ms_g, _ = timed(gemm_alone, K_, W_)
             ms, _ = timed(step_masked, K_, W_)
+        assert ops.static_status(gemm_s, comm_s) == 0, "a device-side wait gave up: the step ran on incomplete tiles"
         print(json.dumps({"steps_only": True, "steps": K_, "warmup": W_, "comm_cus": args.comm_cus,
                           "gemm_cus": cus - args.comm_cus if args.gemm_cus_disjoint else cus,
                           "wave_tiles": fo._capi.wave_tiles(algo, M, N), "cseg": cseg,

@@ -61,8 +61,10 @@ SIGNATURES = {
     "fo_overlap_gemm_allreduce_serial": (c_int, [vp, c_int, c_int, c_int, c_int, vp, vp, vp, c_int]),
     "fo_overlap_seg_allreduce": (c_int, [vp, c_int, vp, c_i64, vp, c_int, c_int]),
     "fo_gemm_set_cu_limit": (c_int, [c_int]),
+    "fo_gemm_set_row_waves": (c_int, [c_int]),
     "fo_gemm_allreduce_overlap_static": (c_int, [c_int, c_int, c_int, c_int, vp, vp, vp, vp, vp, c_int, c_int, c_int,
                                                  vp, vp, c_int, c_int, c_int, vp, vp]),
+    "fo_static_status": (c_int, [vp, vp, vp]),
 }
 
 _lib = None
@@ -136,6 +138,12 @@ def set_gemm_cu_limit(n):
     """The GEMM launches count on n CUs from here on (0: on all); the schedule order, wave_tiles and
     kernel_info answer for that number, so take them again afterwards."""
     check(lib().fo_gemm_set_cu_limit(int(n)), "fo_gemm_set_cu_limit")
+
+
+def set_row_waves(on):
+    """Raster of the 256x256 launches: waves of whole tile rows where they fit (default) or panels only;
+    the schedule order answers for the choice, so take it again afterwards."""
+    check(lib().fo_gemm_set_row_waves(int(bool(on))), "fo_gemm_set_row_waves")
 
 
 def wave_tiles(algo, M, N, dtype=F16):

@@ -1,4 +1,5 @@
 // Algo index space, raster choice and the analytic tile issue order.
+#include <atomic>
 #include <mutex>
 
 #include "fo_common.h"
@@ -8,6 +9,7 @@ namespace {
 fo_algo_entry g_table[128];
 int g_count = 0;
 std::once_flag g_once;
+std::atomic<bool> g_row_waves{true};
 
 // Same enumeration rule as the reference generator (tool/generate_instances.py:5-37):
 // nested product with TbM slowest and Swizzle fastest, minus the shapes CUTLASS
@@ -81,7 +83,39 @@ int fo_pick_raster(int algo, int M, int N, fo_raster *r) {
             r->tail_sub_m = 256 / bm;
             r->tail_sub_n = 256 / bn;
         }
+        // Waves of whole tile rows (fo_row_wave_tile) when the tiles are whole waves and a wave is whole rows
+        // that split into 8 power-of-two blocks; otherwise the panels above.
+        const int per_xcd = resident / 8;
+        if (g_row_waves.load(std::memory_order_relaxed) && r->xcd_remap && rem == 0 && resident % 8 == 0 &&
+            per_xcd > 0 && (per_xcd & (per_xcd - 1)) == 0 && (r->grid_n & (r->grid_n - 1)) == 0) {
+            int log_per = 0, log_gn = 0;
+            while ((1 << log_per) < per_xcd) log_per++;
+            while ((1 << log_gn) < r->grid_n) log_gn++;
+            // blocks as close to square as the row length allows: block width 2^log_bw, 2^log_xc blocks per row
+            int best = -1, best_cost = 0;
+            for (int log_xc = 0; log_xc <= 3; log_xc++) {
+                const int log_bw = log_gn - log_xc, log_bh = log_per - log_bw;
+                if (log_bw < 0 || log_bh < 0) continue;
+                const int cost = (1 << log_bh) + (1 << log_bw);  // operand panels an XCD reads per K step
+                if (best < 0 || cost < best_cost || (cost == best_cost && log_bw > log_bh)) {
+                    best = log_xc;
+                    best_cost = cost;
+                }
+            }
+            if (best >= 0) {
+                const int log_bw = log_gn - best, log_bh = log_per - log_bw;
+                r->xcd_remap = 2;
+                r->panel = fo_pack_row_waves(log_bh, log_bw, best, resident);
+            }
+        }
     }
+    return FO_OK;
+}
+
+void fo_set_row_waves(bool on) { g_row_waves.store(on, std::memory_order_relaxed); }
+
+extern "C" int fo_gemm_set_row_waves(int on) {
+    fo_set_row_waves(on != 0);
     return FO_OK;
 }
 

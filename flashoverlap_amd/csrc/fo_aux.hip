@@ -608,16 +608,17 @@ extern "C" int fo_wait_bounded(int expect, int32_t *counter, int64_t max_polls, 
 // Fills n words; the clearing step of callers that may be under stream capture,
 // where a memset node is avoided.
 namespace {
-__global__ void fo_fill_kernel(int32_t *words, int n, int value) {
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) words[i] = value;
+__global__ void fo_fill_kernel(int32_t *words, int n, int value, int skip) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x)
+        if (i != skip) words[i] = value;
 }
 }  // namespace
 
-int fo_fill_words(int32_t *words, int n, int value, fo_stream_t stream) {
+int fo_fill_words(int32_t *words, int n, int value, fo_stream_t stream, int skip) {
     if (!words || n <= 0) return FO_ERR_ARG;
     const int blocks = (n + 255) / 256;
     hipLaunchKernelGGL(fo_fill_kernel, dim3(blocks < 64 ? blocks : 64), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       words, n, value);
+                       words, n, value, skip);
     FO_LAUNCH_CHECK();
     return FO_OK;
 }

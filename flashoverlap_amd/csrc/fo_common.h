@@ -86,8 +86,8 @@ const fo_algo_entry *fo_algo_lookup(int algo);
 struct fo_raster {
     int mtm, mtn;        // macro tile (workgroup tile) in elements
     int grid_m, grid_n;  // macro tiles along M and N
-    int panel;           // raster panel height in macro tiles
-    int xcd_remap;       // 1: workgroup id is de-interleaved over the 8 XCDs
+    int panel;           // raster panel height in macro tiles (xcd_remap 2: the packed shape of fo_pack_row_waves)
+    int xcd_remap;       // 1: workgroup id is de-interleaved over the 8 XCDs; 2: waves of whole tile rows (below)
     // A last wave of 256x256 tiles that would leave most CUs idle is computed by a
     // second launch instead, with the Algo's own (smaller) tile: the last
     // tail_tiles positions of the raster, each cut into tail_sub_m x tail_sub_n.
@@ -95,6 +95,8 @@ struct fo_raster {
     int resident;  // workgroups of the 256x256 launch the tail split was computed for (0: not a 256x256 raster)
 };
 int fo_pick_raster(int algo, int M, int N, fo_raster *r);
+// Whether fo_pick_raster lays 256x256 launches out in waves of whole tile rows where that fits (default: yes).
+void fo_set_row_waves(bool on);
 // Resident workgroups of the 256x256 kernel shape on the current device (fo_gemm.hip).
 int fo_main_tile_resident();
 
@@ -142,12 +144,34 @@ int fo_wait_reduce_groups_with(int dtype, const void *C, void *ACC, int32_t *MM,
 int fo_wait_with(int expect, int32_t *counter, long max_polls, int32_t *status, fo_stream_t stream);
 int fo_wait_groups_with(int count, const int32_t *expect_dev, int32_t *counters, long max_polls, int32_t *status,
                         fo_stream_t stream);
-// words[0..n) = value by a small kernel (no memset node under stream capture).
-int fo_fill_words(int32_t *words, int n, int value, fo_stream_t stream);
+// words[0..n) = value by a small kernel (no memset node under stream capture); word `skip` keeps its value.
+int fo_fill_words(int32_t *words, int n, int value, fo_stream_t stream, int skip = -1);
+
+// Raster of whole-row waves (xcd_remap == 2).  The persistent launch holds R workgroups, R / 8 on each
+// XCD; wave k of the walk (raster positions kR .. kR + R - 1) covers the R / grid_n complete tile rows
+// that follow those of wave k - 1, cut into 8 blocks of 2^log_bh x 2^log_bw tiles, one per XCD, 2^log_xc
+// blocks side by side: whatever consumes whole output rows (a row-wise normalisation) can follow the GEMM
+// wave by wave.  An XCD's concurrent tiles still form one block and share its operand panels in that
+// XCD's L2.  Everything but the wave index is shifts and masks.
+__host__ __device__ inline int fo_pack_row_waves(int log_bh, int log_bw, int log_xc, int resident) {
+    return log_bh | log_bw << 4 | log_xc << 8 | resident << 12;
+}
+__host__ __device__ inline void fo_row_wave_tile(int t, int packed, int *pm, int *pn) {
+    const int log_bh = packed & 15, log_bw = (packed >> 4) & 15, log_xc = (packed >> 8) & 15, R = packed >> 12;
+    const int k = t / R, w = t - k * R;
+    const int x = w & 7, j = w >> 3;
+    const int rows_per_wave = (8 >> log_xc) << log_bh;
+    *pm = k * rows_per_wave + ((x >> log_xc) << log_bh) + (j & ((1 << log_bh) - 1));
+    *pn = ((x & ((1 << log_xc) - 1)) << log_bw) + (j >> log_bh);
+}
 
 // Workgroup id -> macro tile coordinates; identical code on host and device.
 __host__ __device__ inline void fo_wg_to_tile(int wg, int grid_m, int grid_n, int panel,
                                               int xcd_remap, int *pm, int *pn) {
+    if (xcd_remap == 2) {
+        fo_row_wave_tile(wg, panel, pm, pn);
+        return;
+    }
     int nt = grid_m * grid_n;
     int v = wg;
     if (xcd_remap) {

@@ -573,8 +573,27 @@ extern "C" int fo_gemm_allreduce_overlap_static(int dtype, int M, int N, int K, 
     // The array keeps what the last call on this device left: counters of a call whose
     // bounded wait gave up would still be standing.  Cleared by a kernel, not a memset
     // node, in case the GEMM stream is being captured.
-    rc = fo_fill_words(ws, kWorkspaceWords + G, 0, ctx.gemm_stream);
+    // The give-up word is left standing: fo_static_status reads and clears it.
+    rc = fo_fill_words(ws, kWorkspaceWords + G, 0, ctx.gemm_stream, kWsGaveUp);
     if (rc) return rc;
     return allreduce_overlap(&ctx, dtype, M, N, K, A, B, C, ws + kWorkspaceWords, RA, TM, TN, rLDN, cseg_host,
                              cseg_dev, G, algo, 0);
+}
+
+// Whether a bounded device-side wait of an allocation-free call gave up since the
+// last query on this device.  The calls have no handle to ask; the flag word of the
+// static array is sticky across calls until it is read here.
+extern "C" int fo_static_status(fo_stream_t gemm_stream, fo_stream_t comm_stream, int32_t *gave_up) {
+    if (!gave_up) return FO_ERR_ARG;
+    *gave_up = 0;
+    int32_t *ws = nullptr;
+    int token = 0;
+    int rc = scratch_of_current_device(&ws, &token);
+    if (rc) return rc;
+    FO_HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(gemm_stream)));
+    if (comm_stream != gemm_stream) FO_HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(comm_stream)));
+    FO_HIP_CHECK(hipMemcpy(gave_up, ws + kWsGaveUp, sizeof(int32_t), hipMemcpyDeviceToHost));
+    // A wait that gave up may have left the fork or join word set; both streams are idle now.
+    if (*gave_up) FO_HIP_CHECK(hipMemset(ws, 0, kWorkspaceWords * sizeof(int32_t)));
+    return FO_OK;
 }

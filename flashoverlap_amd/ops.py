@@ -327,3 +327,13 @@ def gemm_allreduce_overlap_static(A, B, C, acc, RA, rLDN, cseg_cpu, cseg_gpu, al
         dtype_code(A), M, N, K, _ptr(A, "A"), _ptr(B, "B"), _ptr(C, "C"), _ptr(acc, "ACC"), _i32(RA, "RA"), TM, TN,
         int(rLDN), _i32(cseg_cpu, "cSEG_CPU", cuda=False), _i32(cseg_gpu, "cSEG_GPU"), cseg_gpu.numel(), int(algo),
         int(fused), gs, cs), "fo_gemm_allreduce_overlap_static")
+
+
+def static_status(gemm_stream=None, comm_stream=None):
+    """Synchronises the streams of the allocation-free calls; 1 if one of their bounded waits gave up
+    since the last query on this device, else 0."""
+    gs = _stream(gemm_stream)
+    cs = gs if comm_stream is None else _stream(comm_stream)
+    out = ctypes.c_int32(0)
+    check(lib().fo_static_status(gs, cs, ctypes.byref(out)), "fo_static_status")
+    return out.value

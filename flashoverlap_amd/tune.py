@@ -218,6 +218,51 @@ def time_overlap(M, N, K, algo, cseg, hint, dtype=torch.float16, warmup=20, reps
     return ms
 
 
+def compare_overlap(M, N, K, algo, csegs, hint, dtype=torch.float16, rounds=2, reps=30, warmup=3,
+                    with_consumer=True):
+    """Median ms of the overlapped call for each cSeg of `csegs`, measured on one set of buffers with
+    the candidates taking turns (`rounds` passes over all of them, `reps` timed calls each): what is
+    left of clock drift and of one-off disturbances falls on all candidates alike.  For deciding
+    between splits that differ by a few percent; time_overlap's mean of one run does not resolve that."""
+    BM, BN = _capi.algo_tile(algo)
+    TM, TN = M // BM, N // BN
+    A = torch.randn(M, K, device="cuda").to(dtype)
+    B = torch.randn(N, K, device="cuda").to(dtype)
+    C = torch.empty(M, N, device="cuda", dtype=dtype)
+    RA = reorder_indices(TM * TN, hint).reshape(TM, TN)
+    MM = torch.zeros(counter_size(max(len(c) for c in csegs), TM, TN), dtype=torch.int32, device="cuda")
+    ov = ops.Overlap()
+    if with_consumer:
+        ov.set_accumulator(torch.zeros(M * N, device="cuda", dtype=dtype))
+    calls = []
+    for cseg in csegs:
+        c_cpu = torch.tensor(cseg, dtype=torch.int32)
+        c_gpu = c_cpu.cuda()
+        if len(cseg) == 1:
+            calls.append(lambda: ov.gemm_allreduce(A, B, C, algo))
+        else:
+            calls.append(lambda c_cpu=c_cpu, c_gpu=c_gpu: ov.gemm_allreduce_overlap(A, B, C, MM, RA, 1, c_cpu, c_gpu, algo))
+    samples = [[] for _ in csegs]
+    _time_ms(calls[0], 0, 1, settle_s=0.3)
+    for _ in range(rounds):
+        for i, fn in enumerate(calls):
+            for _ in range(warmup):
+                fn()
+            start = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
+            end = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
+            for k in range(reps):
+                start[k].record()
+                fn()
+                end[k].record()
+            torch.cuda.synchronize()
+            samples[i] += [s.elapsed_time(e) for s, e in zip(start, end)]
+    gave_up = ov.status()
+    ov.close()
+    if gave_up:
+        raise RuntimeError("a device-side wait gave up while timing the overlapped call")
+    return [float(np.median(x)) for x in samples]
+
+
 def exhaustive_search(M, N, K, algo, wave, hint, dtype=torch.float16, reps=50):
     """Measure every composition of the wave count (tune/search.py:387-439)."""
     BM, BN = _capi.algo_tile(algo)
@@ -230,6 +275,33 @@ def exhaustive_search(M, N, K, algo, wave, hint, dtype=torch.float16, reps=50):
         if ms < best_ms:
             best, best_ms = cseg, ms
     return best, best_ms, table
+
+
+def choose_candidate(M, N, K, BMs, BNs, algos, predictive, dtype=torch.float16, measure=None, wave_of=None,
+                     order_of=None):
+    """Walk down the stage-1 GEMM candidates (the first 5 for the exhaustive search, the first 10 for the
+    predictive one) until monitor mode gives a hint that is consistent with the wave structure, as
+    tune/search.py:397-411 and :452-468 do; the predictive search asks for consistency in units of its
+    smallest group, ceil(waves / 10) waves (:462-465).  Returns (candidate index, hint, consistent).
+    Where the reference gives up ("Tuning fails!"), the first candidate is taken with the order its
+    persistent launch walks the tiles in, which needs no measurement.  A candidate whose group count
+    leaves monitor mode no room for its order counter (groups > TN - 1) cannot be measured and is passed
+    over.  measure / wave_of / order_of default to measured_hint, _capi.wave_tiles and
+    _capi.schedule_order (arguments for tests)."""
+    measure = measure or (lambda algo, wave: measured_hint(M, N, K, algo, wave, dtype))
+    wave_of = wave_of or (lambda algo: _capi.wave_tiles(algo, M, N))
+    order_of = order_of or (lambda algo: _capi.schedule_order(algo, M, N))
+    for t in range(min(10 if predictive else 5, len(algos))):
+        BM, BN, algo = BMs[t], BNs[t], algos[t]
+        tile_num = (M // BM) * (N // BN)
+        wave = wave_of(algo)
+        unit = wave * div_up(div_up(tile_num, wave), 10) if predictive else wave
+        if div_up(tile_num, unit) > N // BN - 1:   # monitor mode keeps its order counter at MM[TN-1]
+            continue
+        ok, hint = measure(algo, unit)
+        if ok:
+            return t, hint, True
+    return 0, order_of(algos[0]), False
 
 
 # ------------------------------------------------------------------ command line
@@ -252,23 +324,19 @@ def tune_shape(M, N, K, comm_op="all_reduce", predictive=False, dtype=torch.floa
         cdir = directory or config.DEFAULT_DIR
         os.makedirs(cdir, exist_ok=True)
         torch.save(curve, os.path.join(cdir, f"bandwidth_{comm_op}_tp1.pt"))
-    BM, BN, dur, algo = BMs[0], BNs[0], durs[0], algos[0]
+    t, hint, consistent = choose_candidate(M, N, K, BMs, BNs, algos, predictive, dtype)
+    BM, BN, dur, algo = BMs[t], BNs[t], durs[t], algos[t]
     tile_num = (M // BM) * (N // BN)
     wave = _capi.wave_tiles(algo, M, N)
-    analytic = _capi.schedule_order(algo, M, N)
-    hint = analytic
-    if div_up(tile_num, wave) <= N // BN - 1:   # monitor mode keeps its order counter at MM[TN-1]
-        ok, measured = measured_hint(M, N, K, algo, wave, dtype)
-        say("monitor-mode hint consistent with the wave structure:", ok)
-        if ok:
-            hint = measured
+    say("GEMM candidate %d (Algo %d, %dx%d): monitor-mode hint consistent with the wave structure: %s"
+        % (t, algo, BM, BN, consistent))
     if predictive:
         cseg, est = predictive_search(M, N, dur, curve.numpy(), tile_num, wave)
         say("predicted latency %.4f ms for cSeg %s" % (est, cseg))
     else:
         cseg, ms, table = exhaustive_search(M, N, K, algo, wave, hint, dtype, reps=max(10, reps // 4))
-        for c, t in table:
-            say(c, "%.4f" % t)
+        for c, c_ms in table:
+            say(c, "%.4f" % c_ms)
     ms = time_overlap(M, N, K, algo, cseg, hint, dtype, warmup=10, reps=reps)
     say("searched latency %.4f ms, best cSeg %s" % (ms, cseg))
     path = config.save_solution(M, N, K, BM, BN, dur, algo, hint, cseg, directory=directory)

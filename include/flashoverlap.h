@@ -88,6 +88,16 @@ int fo_gemm_kernel_info(int dtype, int algo, int M, int N, int epilogue, int32_t
  * changing it.  The reference assumes sm_count - 2 SMs for the GEMM in the same
  * places (tune/search.py:404-407, :459-464, test/test.py:330). */
 int fo_gemm_set_cu_limit(int n);
+/* Raster of the 256x256 launches (no counterpart in the reference, whose tile
+ * order is the hardware scheduler's).  on != 0 (the default): where the tiles are
+ * whole waves of the persistent launch and a wave is whole tile rows that split
+ * into eight power-of-two blocks (one per XCD), wave k computes the tile rows
+ * that follow those of wave k - 1, so that a consumer of whole output rows
+ * (fo_overlap_gemm_allreduce_norm) can follow the GEMM wave by wave; elsewhere,
+ * and with on == 0 everywhere, each XCD walks a panel of the Algo's swizzle
+ * height across all columns.  Process-wide; take fo_schedule_order (and the RA
+ * built from it) again after changing it. */
+int fo_gemm_set_row_waves(int on);
 
 /* ---- GEMM -------------------------------------------------------------
  * C[M,N] = A[M,K] . B[N,K]^T, 16-bit in/out, fp32 accumulate.
@@ -133,11 +143,6 @@ int fo_gemm_scatter(int dtype, int M, int N, int K, int rLDN, const int32_t *cse
  * report it through fo_overlap_status. */
 int fo_wait(int expect, int32_t *counter, fo_stream_t stream);
 
-/* Same, but gives up after max_polls polls (0 = unbounded) and then writes 1
- * to *status (device int32, may be NULL) without touching the counter; on
- * success *status is left unchanged.  No counterpart in the reference (its
- * waiter spins forever); exists so that failure handling can be tested
- * without hanging a GPU. */
 /* fo_wait for `count` consecutive groups in one launch: for every g in
  * 0..count-1 (a lane per group, side by side), spin until counters[g] ==
  * expect_dev[g] (device array, e.g. cSEG_GPU + i), then reset counters[g]; the
@@ -149,6 +154,11 @@ int fo_wait_groups(int count, const int32_t *expect_dev, int32_t *counters, fo_s
  * fo_set complete (and visible) before the word changes, and the waiting stream continues
  * a few microseconds later -- an event wait across queues measured about 12 us here. */
 int fo_set(int32_t *word, int value, fo_stream_t stream);
+/* fo_wait that gives up after max_polls polls (0 = unbounded) and then writes 1
+ * to *status (device int32, may be NULL) without touching the counter; on
+ * success *status is left unchanged.  No counterpart in the reference (its
+ * waiter spins forever); exists so that failure handling can be tested
+ * without hanging a GPU. */
 int fo_wait_bounded(int expect, int32_t *counter, int64_t max_polls, int32_t *status,
                     fo_stream_t stream);
 
@@ -330,6 +340,12 @@ int fo_gemm_allreduce_overlap_static(int dtype, int M, int N, int K, const void 
                                      void *acc, const int32_t *RA, int TM, int TN, int rLDN,
                                      const int32_t *cseg_host, const int32_t *cseg_dev, int G, int algo,
                                      int fused, fo_stream_t gemm_stream, fo_stream_t comm_stream);
+/* Status of the allocation-free calls on the current device: synchronises both
+ * streams, then *gave_up = 1 if a bounded device-side wait (FO_WAIT_MAX_POLLS)
+ * of any such call ran out of polls since the last query (the consumer then
+ * ran on incomplete tiles), else 0; reading clears the flag.  Allocates
+ * nothing.  The counterpart of fo_overlap_status for calls without a handle. */
+int fo_static_status(fo_stream_t gemm_stream, fo_stream_t comm_stream, int32_t *gave_up);
 
 #ifdef __cplusplus
 }

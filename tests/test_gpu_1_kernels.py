@@ -403,7 +403,10 @@ def test_streaming_forms_give_the_same_bits(fo, dtype):
 @pytest.mark.parametrize("dtype", [F16, BF16])
 def test_reorder_rmsnorm_undoes_the_permutation(fo, oracle, dtype):
     for (bm, bn, M, N, rldn) in [(128, 128, 256, 1024, 1), (128, 256, 256, 4096, 1), (64, 128, 256, 512, 2),
-                                 (16, 128, 64, 8192, 1), (32, 96, 64, 480, 1)]:  # last: BN no power of two
+                                 (16, 128, 64, 8192, 1), (32, 96, 64, 480, 1),   # last: BN no power of two
+                                 # 128 and 96 tiles per row (slots handed out from two registers per lane; rows of
+                                 # more than 8192 elements), 129 tiles per row (beyond the slot registers: general path)
+                                 (16, 128, 32, 16384, 1), (32, 128, 64, 12288, 1), (16, 64, 32, 8256, 1)]:
         TM, TN = M // bm, N // bn
         T = TM * TN
         rng = np.random.default_rng(40)

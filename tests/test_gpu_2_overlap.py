@@ -523,12 +523,18 @@ def test_predictive_search_against_checker_and_measurement(fo, oracle):
     for gp in tune.integer_partitions(8):
         cseg = tune.groups_to_cseg(gp, 256, T)
         times[tuple(cseg)] = tune.time_overlap(M, N, K, algo, cseg, hint, warmup=3, reps=10, settle_s=0.05)
-    t_pred = times[tuple(pred)]
-    t_best = min(times.values())
-    print(f"predictive {pred}: {t_pred:.4f} ms; exhaustive best {min(times, key=times.get)}: {t_best:.4f} ms; "
-          f"worst {max(times.values()):.4f} ms")
-    # margin: 8 % (the splits differ by a few percent on one GPU and ten repetitions scatter by one or two);
-    # the reference accepts its predictive choice without any such check
+    # Ten repetitions per split only rank the field; the verdict comes from the predicted split and the
+    # five fastest of that pass measured again, taking turns, two rounds of thirty calls, medians.
+    finalists = sorted(times, key=times.get)[:5]
+    if tuple(pred) not in finalists:
+        finalists.append(tuple(pred))
+    med = dict(zip(finalists, tune.compare_overlap(M, N, K, algo, [list(c) for c in finalists], hint, rounds=2, reps=30)))
+    t_pred = med[tuple(pred)]
+    t_best = min(med.values())
+    print(f"predictive {pred}: {t_pred:.4f} ms; best of the finalists {min(med, key=med.get)}: {t_best:.4f} ms; "
+          f"first pass: best {min(times.values()):.4f}, worst {max(times.values()):.4f} ms")
+    # margin: 8 % (the splits differ by a few percent on one GPU); the reference accepts its predictive
+    # choice without any such check
     assert t_pred <= 1.08 * t_best
 
 

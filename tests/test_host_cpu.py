@@ -159,6 +159,58 @@ def test_schedule_order_is_a_permutation_with_local_waves(algo, M, N):
             assert len(rows) * len(cols) <= 64
 
 
+@pytest.mark.parametrize("bm,bn,M,N", [(128, 256, 8192, 8192), (256, 128, 8192, 8192), (128, 128, 8192, 4096),
+                                        (128, 128, 2048, 16384), (128, 128, 16384, 2048)])
+def test_waves_of_the_persistent_launch_are_whole_tile_rows(bm, bn, M, N):
+    """Where the 256x256 tiles are whole waves of 256 workgroups and a wave splits into eight power-of-two
+    blocks, wave k of the schedule order is exactly the tile rows that follow wave k - 1's, each XCD
+    (positions x, x + 8, ... of the wave) owning one block of 32 tiles with at most 12 operand panels."""
+    algo = _capi.find_algo(bm, bn, swizzle=4)
+    order = _capi.schedule_order(algo, M, N)
+    TM, TN = M // bm, N // bn
+    assert sorted(order) == list(range(TM * TN))
+    sub = (256 // bm) * (256 // bn)
+    gm, gn = M // 256, N // 256
+    rows_per_wave = 256 // gn
+    wgs = [order[i:i + sub] for i in range(0, len(order), sub)]
+    macro = [((w[0] // TN) * bm // 256, (w[0] % TN) * bn // 256) for w in wgs]
+    for k in range(gm * gn // 256):
+        wave = macro[k * 256:(k + 1) * 256]
+        assert sorted(wave) == [(k * rows_per_wave + i, j) for i in range(rows_per_wave) for j in range(gn)]
+        for x in range(8):
+            mine = wave[x::8]
+            rows, cols = {m for m, _ in mine}, {n for _, n in mine}
+            assert len(rows) * len(cols) == 32 and len(rows) + len(cols) <= 12
+    # the reorder table built from this order stores wave k's tiles in the k-th stretch of slots:
+    # every tile row's last slot lies in its own wave's stretch
+    RA = layout.reorder_indices(TM * TN, order, device="cpu").reshape(TM, TN)
+    per_wave = 256 * sub
+    for tm in range(TM):
+        assert int(RA[tm].max()) // per_wave == int(RA[tm].min()) // per_wave == (tm * bm // 256) // rows_per_wave
+    # switched off: the panels of the Algo's swizzle, where a wave touches every tile row
+    try:
+        _capi.set_row_waves(False)
+        panels = _capi.schedule_order(algo, M, N)
+    finally:
+        _capi.set_row_waves(True)
+    assert sorted(panels) == list(range(TM * TN)) and _capi.schedule_order(algo, M, N) == order
+    if gm > rows_per_wave and gm >= 32:
+        first_wave_rows = {(w[0] // TN) * bm // 256 for w in [panels[i:i + sub] for i in range(0, 256 * sub, sub)]}
+        assert first_wave_rows != set(range(rows_per_wave))
+
+
+def test_row_waves_need_whole_waves_and_power_of_two_rows():
+    """12288 columns are 48 tiles of 256 (no power of two), 8448^2 leaves a partial last wave: both keep the panels."""
+    for bm, bn, M, N in ((128, 128, 4096, 12288), (128, 128, 8448, 8448)):
+        algo = _capi.find_algo(bm, bn, swizzle=4)
+        order = _capi.schedule_order(algo, M, N)
+        try:
+            _capi.set_row_waves(False)
+            assert _capi.schedule_order(algo, M, N) == order
+        finally:
+            _capi.set_row_waves(True)
+
+
 def test_latency_model_and_search_agree_with_checker(oracle):
     curve = np.array([[2.0 ** (20 + 0.25 * i), 0.5 + 0.1 * i] for i in range(36)])
     M = N = 8192
@@ -175,6 +227,48 @@ def test_latency_model_and_search_agree_with_checker(oracle):
     cands = [tune.groups_to_cseg(gp, wave, tiles) for gp in tune.integer_partitions(8)
              if not (len(gp) > 5 and gp[0] > 2)]
     assert dur == pytest.approx(min(tune.predict_latency(M, N, 0.7, curve, c, tiles, wave) for c in cands))
+
+
+def test_tuner_walks_down_the_gemm_candidates_until_a_hint_is_consistent():
+    """tune/search.py:397-411 (exhaustive: 5 candidates) and :452-468 (predictive: 10, consistency asked in
+    units of ceil(waves/10) waves): the first candidate whose monitor-mode hint is consistent is taken with
+    that hint; if none is, the first candidate with the order its launch walks the tiles in."""
+    M = N = 4096
+    K = 512
+    BMs, BNs = [128] * 12, [128] * 12
+    algos = list(range(100, 112))
+    asked = []
+
+    def measure_ok_from(first_ok):
+        def measure(algo, unit):
+            asked.append((algo, unit))
+            return algo >= first_ok, [algo]
+        return measure
+
+    kw = dict(wave_of=lambda algo: 256, order_of=lambda algo: ["walk", algo])
+    # 1024 tiles, 4 waves of 256: exhaustive consistency unit = one wave
+    t, hint, ok = tune.choose_candidate(M, N, K, BMs, BNs, algos, False, measure=measure_ok_from(103), **kw)
+    assert (t, hint, ok) == (3, [103], True) and asked == [(100, 256), (101, 256), (102, 256), (103, 256)]
+    asked.clear()
+    t, hint, ok = tune.choose_candidate(M, N, K, BMs, BNs, algos, False, measure=measure_ok_from(105), **kw)
+    assert (t, hint, ok) == (0, ["walk", 100], False) and len(asked) == 5      # only five are tried
+    asked.clear()
+    t, hint, ok = tune.choose_candidate(M, N, K, BMs, BNs, algos, True, measure=measure_ok_from(109), **kw)
+    assert (t, hint, ok) == (9, [109], True) and len(asked) == 10
+    asked.clear()
+    t, hint, ok = tune.choose_candidate(M, N, K, BMs, BNs, algos, True, measure=measure_ok_from(110), **kw)
+    assert (t, hint, ok) == (0, ["walk", 100], False) and len(asked) == 10     # only ten are tried
+    # predictive unit: 40 waves of 26 tiles -> smallest group ceil(40 / 10) = 4 waves = 104 tiles
+    asked.clear()
+    tune.choose_candidate(M, N, K, BMs, BNs, algos, True, measure=measure_ok_from(100), wave_of=lambda a: 26,
+                          order_of=kw["order_of"])
+    assert asked == [(100, 104)]
+    # a candidate that leaves monitor mode no counter for its order stamp is passed over:
+    # 1024 tiles in waves of 16 = 64 groups > TN - 1 = 31; the next candidate (waves of 256) is measured
+    asked.clear()
+    t, _, ok = tune.choose_candidate(M, N, K, BMs, BNs, algos, False, measure=measure_ok_from(100),
+                                     wave_of=lambda a: 16 if a == 100 else 256, order_of=kw["order_of"])
+    assert (t, ok) == (1, True) and asked == [(101, 256)]
 
 
 def test_config_json_two_stage_round_trip(tmp_path):

@@ -41,11 +41,15 @@ def _case(fo, M, N, K, bm, bn, cseg, fused, two_streams, seed):
     C = torch.full((M * N,), float("nan"), device="cuda", dtype=torch.float16)
     acc = acc0.clone()
     comm = torch.cuda.Stream() if two_streams else None
+    fo.ops.static_status(comm_stream=comm)       # first use of the library's static array happens here, not below
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
+    free_before = torch.cuda.mem_get_info()[0]   # the driver's free bytes: sees a hipMalloc that torch's allocator would not
     fo.ops.gemm_allreduce_overlap_static(A, B, C, acc, RA, 1, cs_cpu, cs_gpu, algo, fused=fused, comm_stream=comm)
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] >= free_before   # nothing was taken from the device's memory
+    assert fo.ops.static_status(comm_stream=comm) == 0   # no bounded wait gave up
     assert torch.equal(C, C_ref)                 # reordered tiles: bit-exact
     assert torch.equal(acc, acc_ref)             # consumer: bit-exact
     plain = torch.empty(M, N, device="cuda", dtype=torch.float16)
