@@ -2,7 +2,7 @@
 
 A step = one pass of the hot path over one synthetic batch: GEMM + tile signal +
 reordered store on the GEMM stream, per-group wait + consumer on the second
-stream, join, reorder+RMSNorm.  Workload: the large-square configuration the
+stream followed there by reorder+RMSNorm of the rows each wave completed, join.  Workload: the large-square configuration the
 headline metric is quoted on (fp16, M=N=K=8192, 128x256 tiles, wave groups of
 256 tiles).  Prints one JSON line; `value` is GEMM flops / step time.
 
@@ -101,11 +101,19 @@ def measure(args, workload, compact=False):
         else:
             ops.reorder_rmsnorm(Cp.view(M, N), Y, gamma, BM, BN, 1, RA, eps=eps)
 
+    RA_cpu = RA.cpu()
+
     def step_overlapped():
+        # all-reduce layout: one call, the rows normalised on the consumer stream behind each wave's consumer;
+        # reduce-scatter layout: the overlapped call, then the normalisation of segment 0
         if W:
             ov.gemm_reducescatter_overlap(A, B, Cp, D, MM, RA, RE, 1, cs_cpu, cs_gpu, algo)
+            norm()
         else:
-            ov.gemm_allreduce_overlap(A, B, Cp, MM, RA, 1, cs_cpu, cs_gpu, algo)
+            ov.gemm_allreduce_rmsnorm_overlap(A, B, Cp, MM, RA, RA_cpu, 1, cs_cpu, cs_gpu, algo, Y, gamma, eps=eps)
+
+    def step_pair():  # the reference's two calls: overlapped GEMM + collective, then reorder_rmsnorm behind the join
+        ov.gemm_allreduce_overlap(A, B, Cp, MM, RA, 1, cs_cpu, cs_gpu, algo)
         norm()
 
     def step_serial():  # signal-free GEMM, whole-C consumer, plain RMSNorm, one stream
@@ -201,14 +209,27 @@ def measure(args, workload, compact=False):
         print(json.dumps({"kernels_only": True, "steps": K_, "warmup": W_}))
         return
     settle(step_serial, 0.25 if compact else 0.5)
-    ms_step, wall_step = timed(step_overlapped, K_, W_)
-    ms_serial, _ = timed(step_serial, K_, W_)
-    # second pass in the opposite order: what remains of drift between the two shows up here
-    ms_serial2, _ = timed(step_serial, K_, W_)
-    ms_step2, _ = timed(step_overlapped, K_, W_)
-    ms_gemm, _ = timed(gemm_alone, K_, W_)
-    ms_signal, _ = timed(gemm_signal_alone, K_, W_)
-    MM.zero_()
+    # The ratios asked for are differences of one to ten percent between runs that drift by as much over a
+    # second: overlapped step, serial step, GEMM alone and signal GEMM take turns in `blocks` rounds of
+    # W_ + K_ launches each, and every figure is the median of its blocks.
+    import statistics
+    blocks = 3 if compact else args.blocks
+    legs = {"overlapped": step_overlapped, "serial": step_serial, "gemm": gemm_alone, "signal": gemm_signal_alone}
+    if not W:
+        legs["pair"] = step_pair
+    samples = {k: [] for k in legs}
+    wall_step = 0.0
+    for _ in range(blocks):
+        for name, fn in legs.items():
+            ms, wall = timed(fn, K_, W_)
+            samples[name].append(ms)
+            if name == "overlapped":
+                wall_step = wall
+            if name == "signal":
+                MM.zero_()
+    med = {k: statistics.median(v) for k, v in samples.items()}
+    ms_step, ms_serial, ms_gemm, ms_signal = med["overlapped"], med["serial"], med["gemm"], med["signal"]
+    ms_pair = med.get("pair")
     # the vendor library's GEMM on the same operands, same process and clocks: a yardstick only
     def vendor_gemm():
         torch.matmul(A, B.t(), out=Cplain)
@@ -224,7 +245,7 @@ def measure(args, workload, compact=False):
         ov.close()
         return {"workload": f"{workload}: {desc}", "dtype": dt, "cseg": cseg if len(cseg) <= 16 else f"{len(cseg)} x {cseg[0]}",
                 "gemm_alone_ms": ms_gemm, "gemm_signal_ms": ms_signal, "frac": flops / (ms_signal * 1e-3) / 1e12 / PEAK_TFLOPS,
-                "overlapped_ms": ms_step, "serial_ms": ms_serial,
+                "overlapped_ms": ms_step, "serial_ms": ms_serial, "two_calls_ms": ms_pair, "blocks": blocks,
                 "overlapped_vs_gemm_alone": ms_step / ms_gemm, "overlapped_vs_serial": ms_step / ms_serial,
                 "consumer_GBps": 6.0 * M * N / (ms_consumer * 1e-3) / 1e9,
                 "reorder_rmsnorm_GBps": (4.0 * bs * N + 2.0 * N) / (ms_norm * 1e-3) / 1e9,
@@ -243,8 +264,7 @@ def measure(args, workload, compact=False):
             c_gpu = c_cpu.cuda()
 
             def step_g():
-                ov.gemm_allreduce_overlap(A, B, Cp, MM, RA, 1, c_cpu, c_gpu, algo)
-                norm()
+                ov.gemm_allreduce_rmsnorm_overlap(A, B, Cp, MM, RA, RA_cpu, 1, c_cpu, c_gpu, algo, Y, gamma, eps=eps)
             ms_g, _ = timed(step_g, K_, W_)
             sweep.append({"waves_per_group": waves, "groups": len(cs), "ms": ms_g, "path": "overlapped",
                           "vs_serial": ms_g / ms_serial, "vs_gemm_alone": ms_g / ms_gemm})
@@ -263,8 +283,7 @@ def measure(args, workload, compact=False):
         ov.set_accumulator(ACCb)
 
         def step_b():
-            ov.gemm_allreduce_overlap(Ab, Bb, Cb, MM, RA, 1, cs_cpu, cs_gpu, algo)
-            ops.reorder_rmsnorm(Cb.view(M, N), Yb, gb, BM, BN, 1, RA, eps=eps)
+            ov.gemm_allreduce_rmsnorm_overlap(Ab, Bb, Cb, MM, RA, RA_cpu, 1, cs_cpu, cs_gpu, algo, Yb, gb, eps=eps)
 
         def serial_b():
             ops.gemm(Ab, Bb, Cbp, algo)
@@ -274,10 +293,13 @@ def measure(args, workload, compact=False):
         def signal_b():
             ops.gemm_signal(Ab, Bb, Cb, MM, RA, cs_gpu, algo)
         settle(serial_b, 0.3)  # the allocations above left the GPU idle
-        ms_b, _ = timed(step_b, K_, W_)
-        ms_sb, _ = timed(serial_b, K_, W_)
-        ms_gb, _ = timed(signal_b, K_, W_)
-        MM.zero_()
+        sb = {"step": [], "serial": [], "signal": []}
+        for _ in range(3):
+            sb["step"].append(timed(step_b, K_, W_)[0])
+            sb["serial"].append(timed(serial_b, K_, W_)[0])
+            sb["signal"].append(timed(signal_b, K_, W_)[0])
+            MM.zero_()
+        ms_b, ms_sb, ms_gb = (statistics.median(sb[k]) for k in ("step", "serial", "signal"))
         torch.cuda.synchronize()
         bf16_repeat = {"overlapped_step_ms": ms_b, "serial_step_ms": ms_sb, "gemm_signal_alone_ms": ms_gb,
                        "gemm_signal_TFLOPs": 2.0 * M * N * K / (ms_gb * 1e-3) / 1e12,
@@ -310,12 +332,14 @@ def measure(args, workload, compact=False):
                      if (workload, dt) in MEASURED_TRAFFIC_BYTES else None},
         "times_ms": {"overlapped_step": ms_step, "overlapped_step_wall": wall_step,
                      "serial_step": ms_serial, "gemm_alone": ms_gemm, "gemm_signal_alone": ms_signal,
+                     "two_calls_step": ms_pair,
                      "consumer_alone": ms_consumer, "reorder_rmsnorm_alone": ms_norm,
                      "vendor_gemm_torch_matmul": ms_vendor},
         "overlapped_vs_gemm_alone": ms_step / ms_gemm,
         "overlapped_vs_serial": ms_step / ms_serial,
-        "second_pass_ms": {"serial_step": ms_serial2, "overlapped_step": ms_step2,
-                           "overlapped_vs_serial": ms_step2 / ms_serial2},
+        "two_calls_vs_serial": ms_pair / ms_serial if ms_pair else None,
+        "timing": {"blocks": blocks, "steps_per_block": K_, "warmup_per_block": W_, "figure": "median of the blocks",
+                   "block_ms": {k: [round(x, 4) for x in v] for k, v in samples.items()}},
         "consumer_GBps": 6.0 * M * N / (ms_consumer * 1e-3) / 1e9,
         "reorder_rmsnorm_GBps": (4.0 * bs * N + 2.0 * N) / (ms_norm * 1e-3) / 1e9,
         "hbm_peak_GBps": PEAK_HBM_GBS,
@@ -332,6 +356,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--blocks", type=int, default=5,
+                    help="rounds in which the overlapped step, the serial step and the two GEMMs take turns "
+                         "(warmup + steps launches each per round); every reported time is the median of its blocks")
     ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS))
     ap.add_argument("--dtype", default=None, choices=["f16", "bf16"])
     ap.add_argument("--swizzle", type=int, default=4)

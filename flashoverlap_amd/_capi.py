@@ -40,6 +40,8 @@ SIGNATURES = {
                                       c_int, c_int, c_int, vp]),
     "fo_reorder_rmsnorm": (c_int, [c_int, vp, vp, vp, c_int, c_int, c_int, c_int, c_int, vp, c_f32,
                                    vp]),
+    "fo_reorder_rmsnorm_rows": (c_int, [c_int, vp, vp, vp, c_int, c_int, c_int, c_int, c_int, c_int, c_int, vp, c_f32,
+                                        vp]),
     "fo_rmsnorm": (c_int, [c_int, vp, vp, vp, c_int, c_int, c_f32, vp]),
     "fo_overlap_plan_batches": (c_int, [vp, c_int, c_int, vp]),
     "fo_overlap_create": (c_int, [ctypes.POINTER(vp)]),
@@ -56,6 +58,8 @@ SIGNATURES = {
     "fo_overlap_gemm": (c_int, [vp, c_int, c_int, c_int, c_int, vp, vp, vp, c_int]),
     "fo_overlap_gemm_allreduce": (c_int, [vp, c_int, c_int, c_int, c_int, vp, vp, vp, vp, vp, c_int,
                                           c_int, c_int, vp, vp, c_int, c_int, c_int]),
+    "fo_overlap_gemm_allreduce_norm": (c_int, [vp, c_int, c_int, c_int, c_int, vp, vp, vp, vp, vp, vp, c_int,
+                                               c_int, c_int, vp, vp, c_int, c_int, c_int, vp, vp, c_f32]),
     "fo_overlap_gemm_reducescatter": (c_int, [vp, c_int, c_int, c_int, c_int, vp, vp, vp, vp, vp, vp,
                                               vp, c_int, c_int, c_int, vp, vp, c_int, c_int, c_int]),
     "fo_overlap_gemm_allreduce_serial": (c_int, [vp, c_int, c_int, c_int, c_int, vp, vp, vp, c_int]),

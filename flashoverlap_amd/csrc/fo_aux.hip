@@ -540,6 +540,200 @@ int launch_rmsnorm(const void *X, void *Y, const void *Wt, int bs, int dim, int 
     return launch_rmsnorm_as<Tag, false>(X, Y, Wt, bs, dim, BM, BN, rldn, RA, eps, stream);
 }
 
+// The same arithmetic for a range of rows, built to run beside a GEMM that holds every CU: one
+// workgroup of four wavefronts works on one row at a time (lane t of the workgroup owns chunks t,
+// t + 256, ...), so a row costs a lane CH x 4 registers instead of MAXCH x 4, the weight chunks stay
+// in registers for all of the workgroup's rows, and the only LDS is eight partial sums.  One such
+// workgroup fits into what a 256x256 GEMM workgroup leaves of a CU (the kernel above needs 16 KiB of
+// LDS and about 100 registers for rows of 8192, and would wait for the GEMM to end).  A workgroup
+// takes consecutive rows; the next row's chunks are requested before the current row is reduced,
+// scaled and stored.  Addresses are buffer-relative: a chunk's byte offset inside its tile row's
+// stretch of the reordered matrix is computed (and its tile's storage slot fetched) only when the
+// rows move on to the next tile row, the row inside the tile is a scalar offset, and the output
+// row's base is a scalar too, so a row costs a lane CH loads, CH stores and no address arithmetic.
+// The matrix must lie within 4 GiB (32-bit byte offsets).
+// Registers: up to 96 per lane, which is what the signalling GEMM's wavefront leaves of its SIMD's
+// 512 (at most 408 with the accumulators); rows above 8192 elements (CH = 8) do without the look-ahead
+// and may take 128, which fits beside the plain GEMM's wavefront only.
+template <typename Tag, int CH, bool STREAM, int PATH>
+__global__ __launch_bounds__(256, CH <= 4 ? 5 : 4) void fo_norm_rows_kernel(const fo_u32x4 *X, fo_u32x4 *Y, const fo_u32x4 *Wt,
+                                                              int row0, int nrows, int rows_per_wg, int dim, int BM,
+                                                              int BN, int rldn, const int32_t *RA, float eps,
+                                                              unsigned x_bytes) {
+    typedef norm_math<Tag> MATH;
+    __shared__ float part[2][4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int nch = dim >> 3;
+    const bool full = nch == 256 * CH;
+    const int first = row0 + blockIdx.x * rows_per_wg;
+    const int last = first + rows_per_wg < row0 + nrows ? first + rows_per_wg : row0 + nrows;
+    if (first >= last) return;
+    constexpr int NT = STREAM ? 2 : 0;  // cache policy bits of the buffer instructions: non-temporal
+    auto chunk_of = [&](int i) {  // this lane's i-th chunk, clamped into the row
+        const int c = tid + i * 256;
+        return c < nch ? c : nch - 1;
+    };
+    fo_u32x4 w[CH];
+#pragma unroll
+    for (int i = 0; i < CH; i++) w[i] = Wt[chunk_of(i)];
+    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)X, 0, x_bytes, 0x00027000);
+    const int ldn = PATH == NORM_PLAIN ? 0 : dim / BN;
+    const int bn_shift = PATH == NORM_SLOTS ? __builtin_ctz(BN) : 0;
+    const unsigned ldp_bytes = (unsigned)rldn * BN * 2;  // row pitch of the reordered view
+    unsigned off[CH];  // byte offset of this lane's chunks in row 0 of their tiles (PLAIN: in the row)
+#pragma unroll
+    for (int i = 0; i < CH; i++) off[i] = (unsigned)chunk_of(i) * 16u;
+    int slot_row = -1;
+    auto request = [&](int b, fo_u32x4(&x)[CH]) {
+        unsigned row_off;  // wave-uniform
+        if (PATH == NORM_PLAIN) {
+            row_off = (unsigned)b * (unsigned)dim * 2u;
+        } else {
+            const int tile_row = b / BM, in_row = b - tile_row * BM;
+            if (tile_row != slot_row) {  // the same for every lane of the workgroup
+#pragma unroll
+                for (int i = 0; i < CH; i++) {
+                    const int j = chunk_of(i) << 3;
+                    const int r = RA[(long)tile_row * ldn + (PATH == NORM_SLOTS ? j >> bn_shift : j / BN)];
+                    if (PATH == NORM_SLOTS)
+                        off[i] = ((unsigned)r * BM << (bn_shift + 1)) + (unsigned)(j & (BN - 1)) * 2u;
+                    else
+                        off[i] = (unsigned)(r / rldn) * BM * ldp_bytes + (unsigned)((r % rldn) * BN + j % BN) * 2u;
+                }
+                slot_row = tile_row;
+            }
+            row_off = (unsigned)in_row * ldp_bytes;
+        }
+        row_off = __builtin_amdgcn_readfirstlane(row_off);
+#pragma unroll
+        for (int i = 0; i < CH; i++)
+            x[i] = __builtin_bit_cast(fo_u32x4, __builtin_amdgcn_raw_buffer_load_b128(xr, off[i], row_off, NT));
+    };
+
+    // One row: reduce, meet, scale, store.
+    int buf = 0;
+    auto finish = [&](int b, fo_u32x4(&x)[CH]) {
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            const float with = MATH::sumsq(x[i], ss);
+            ss = (full || tid + i * 256 < nch) ? with : ss;
+        }
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) ss += __shfl_xor(ss, d, 64);
+        if (lane == 0) part[buf][wave] = ss;
+        __syncthreads();
+        // Two sets of partial sums: a wavefront that runs ahead writes the next row's into the other
+        // set, and cannot reach the row after that before every wavefront has passed the next barrier.
+        const float total = (part[buf][0] + part[buf][1]) + (part[buf][2] + part[buf][3]);
+        buf ^= 1;
+        const float s = rsqrtf(total / (float)dim + eps);
+        // The output row as a buffer of its own: scalar base, the lane's chunks at tid * 16 + i * 4096; chunks beyond
+        // the row's end are out of the buffer's range and the hardware drops their stores.  The stores are
+        // assembly for two reasons.  The compiler counts loads and stores in one counter and, with both kinds in
+        // flight, waits for everything before it touches a loaded register: the next row would never be on its
+        // way during this one.  And a 16-byte store's data registers are read for some cycles after it issues, so
+        // a vector instruction that writes one of them right behind it must keep two wait states; the compiler
+        // leaves them out for the buffer form with a scalar offset register, and lanes 12-63 of a stored chunk
+        // then carried the next chunk's intermediate values whenever the CU was busy.
+        const uint64_t yb = (uint64_t)(uintptr_t)(Y + (long)b * nch);
+        fo_u32x4 yr;
+        yr.x = __builtin_amdgcn_readfirstlane((unsigned)yb);
+        yr.y = __builtin_amdgcn_readfirstlane((unsigned)(yb >> 32) & 0xFFFF);
+        yr.z = __builtin_amdgcn_readfirstlane((unsigned)nch * 16u);
+        yr.w = 0x00027000u;
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            const fo_u32x4 y = MATH::scale(x[i], s, w[i]);
+            if (STREAM)
+                asm volatile("buffer_store_dwordx4 %0, %1, %2, %3 offen nt\n\ts_nop 1"
+                             :
+                             : "v"(y), "v"((unsigned)tid * 16u), "s"(yr), "s"(i * 4096)
+                             : "memory");
+            else
+                asm volatile("buffer_store_dwordx4 %0, %1, %2, %3 offen\n\ts_nop 1"
+                             :
+                             : "v"(y), "v"((unsigned)tid * 16u), "s"(yr), "s"(i * 4096)
+                             : "memory");
+        }
+    };
+
+    // Rows take turns in two register sets, so the row after the one being finished is already on its way.
+    constexpr bool AHEAD = CH <= 4;
+    fo_u32x4 xa[CH], xb[AHEAD ? CH : 1];
+    if (!AHEAD) {
+        for (int b = first; b < last; b++) {
+            request(b, xa);
+            finish(b, xa);
+        }
+        return;
+    }
+    // The loop body holds no branch around a request: where paths with and without a request in flight
+    // meet, the compiler waits as if there were none, i.e. for everything.  The last one or two rows follow it.
+    fo_u32x4(&xb_)[CH] = reinterpret_cast<fo_u32x4(&)[CH]>(xb);
+    request(first, xa);
+    int b = first;
+    for (; b + 2 < last; b += 2) {
+        request(b + 1, xb_);
+        finish(b, xa);
+        request(b + 2, xa);
+        finish(b + 1, xb_);
+    }
+    if (b + 1 < last) {
+        request(b + 1, xb_);
+        finish(b, xa);
+        finish(b + 1, xb_);
+    } else {
+        finish(b, xa);
+    }
+}
+
+// grid <= 0: one workgroup per 4 rows, at most 2048.  beside_gemm: at most 256 workgroups, each asking for
+// kBesideGemmLds bytes of LDS it never touches (one workgroup per CU beside the GEMM's, as for the consumer).
+template <typename Tag, bool STREAM, int PATH>
+int launch_norm_rows_on(const void *X, void *Y, const void *Wt, int row0, int nrows, int dim, int BM, int BN, int rldn,
+                        const int32_t *RA, float eps, bool beside_gemm, int grid, unsigned x_bytes, hipStream_t stream) {
+    const int nch = dim / 8;
+    if (grid <= 0) grid = (nrows + 3) / 4;
+    const int most = beside_gemm ? 256 : 2048;
+    if (grid > most) grid = most;
+    const int rows_per_wg = (nrows + grid - 1) / grid;
+    grid = (nrows + rows_per_wg - 1) / rows_per_wg;
+    const int lds = beside_gemm ? kBesideGemmLds : 0;
+    const fo_u32x4 *x = static_cast<const fo_u32x4 *>(X);
+    fo_u32x4 *y = static_cast<fo_u32x4 *>(Y);
+    const fo_u32x4 *w = static_cast<const fo_u32x4 *>(Wt);
+#define FO_NORM_ROWS(CH_)                                                                                          \
+    hipLaunchKernelGGL((fo_norm_rows_kernel<Tag, CH_, STREAM, PATH>), dim3(grid), dim3(256), lds, stream, x, y, w, row0, \
+                       nrows, rows_per_wg, dim, BM, BN, rldn, RA, eps, x_bytes)
+    if (nch <= 256)
+        FO_NORM_ROWS(1);
+    else if (nch <= 512)
+        FO_NORM_ROWS(2);
+    else if (nch <= 1024)
+        FO_NORM_ROWS(4);
+    else if (nch <= 2048)
+        FO_NORM_ROWS(8);
+    else
+        return FO_ERR_SHAPE;
+#undef FO_NORM_ROWS
+    FO_LAUNCH_CHECK();
+    return FO_OK;
+}
+
+template <typename Tag, bool STREAM>
+int launch_norm_rows_as(const void *X, void *Y, const void *Wt, int row0, int nrows, int dim, int BM, int BN, int rldn,
+                        const int32_t *RA, float eps, bool beside_gemm, int grid, unsigned x_bytes, hipStream_t stream) {
+    if (!RA)
+        return launch_norm_rows_on<Tag, STREAM, NORM_PLAIN>(X, Y, Wt, row0, nrows, dim, BM, BN, rldn, RA, eps, beside_gemm,
+                                                            grid, x_bytes, stream);
+    if (rldn == 1 && (BN & (BN - 1)) == 0)
+        return launch_norm_rows_on<Tag, STREAM, NORM_SLOTS>(X, Y, Wt, row0, nrows, dim, BM, BN, rldn, RA, eps, beside_gemm,
+                                                            grid, x_bytes, stream);
+    return launch_norm_rows_on<Tag, STREAM, NORM_GENERAL>(X, Y, Wt, row0, nrows, dim, BM, BN, rldn, RA, eps, beside_gemm,
+                                                          grid, x_bytes, stream);
+}
+
 // FO_WAIT_MAX_POLLS (environment, read once): bound for the otherwise unbounded
 // waits, so that a missing signal ends in a flagged exit instead of a hung GPU.
 long default_max_polls() {
@@ -768,6 +962,45 @@ extern "C" int fo_reorder_rmsnorm(int dtype, const void *X, void *Y, const void 
     if (dtype == FO_F16) return launch_rmsnorm<fo_f16_tag>(X, Y, Wt, bs, dim, BM, BN, rldn, RA, eps, s);
     if (dtype == FO_BF16) return launch_rmsnorm<fo_bf16_tag>(X, Y, Wt, bs, dim, BM, BN, rldn, RA, eps, s);
     return FO_ERR_DTYPE;
+}
+
+int fo_norm_rows_with(int dtype, const void *X, void *Y, const void *Wt, int row0, int nrows, int bs, int dim, int BM,
+                      int BN, int rldn, const int32_t *RA, float eps, bool stream_rows, bool beside_gemm, int grid,
+                      fo_stream_t stream) {
+    if (!X || !Y || !Wt || bs <= 0 || dim <= 0 || BM <= 0 || BN <= 0 || rldn <= 0) return FO_ERR_ARG;
+    if (row0 < 0 || nrows < 0 || row0 + nrows > bs) return FO_ERR_ARG;
+    if (dim % 8 || dim > 16384) return FO_ERR_SHAPE;
+    if (RA) {
+        if (BN % 8 || dim % BN || bs % BM) return FO_ERR_SHAPE;
+        if (((long)(bs / BM) * (dim / BN)) % rldn) return FO_ERR_SHAPE;
+    }
+    if ((int64_t)bs * dim * 2 > 0xFFFFFFFFLL) return FO_ERR_SHAPE;  // 32-bit byte offsets into X
+    if (nrows == 0) return FO_OK;
+    const unsigned x_bytes = (unsigned)((int64_t)bs * dim * 2);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == FO_F16)
+        return stream_rows ? launch_norm_rows_as<fo_f16_tag, true>(X, Y, Wt, row0, nrows, dim, BM, BN, rldn, RA, eps, beside_gemm, grid, x_bytes, s)
+                           : launch_norm_rows_as<fo_f16_tag, false>(X, Y, Wt, row0, nrows, dim, BM, BN, rldn, RA, eps, beside_gemm, grid, x_bytes, s);
+    if (dtype == FO_BF16)
+        return stream_rows ? launch_norm_rows_as<fo_bf16_tag, true>(X, Y, Wt, row0, nrows, dim, BM, BN, rldn, RA, eps, beside_gemm, grid, x_bytes, s)
+                           : launch_norm_rows_as<fo_bf16_tag, false>(X, Y, Wt, row0, nrows, dim, BM, BN, rldn, RA, eps, beside_gemm, grid, x_bytes, s);
+    return FO_ERR_DTYPE;
+}
+
+extern "C" int fo_reorder_rmsnorm_rows(int dtype, const void *X, void *Y, const void *Wt, int row0, int nrows, int bs,
+                                       int dim, int BM, int BN, int rldn, const int32_t *RA, float eps,
+                                       fo_stream_t stream) {
+    static const int grid = [] {
+        const char *e = getenv("FO_NORM_GRID");
+        return e ? atoi(e) : 0;
+    }();
+    static const int nt = [] {
+        const char *e = getenv("FO_NORM_NT");
+        return e ? atoi(e) : -1;
+    }();
+    const bool stream_rows = nt < 0 ? fo_streams((int64_t)bs * dim * 4) : nt != 0;
+    return fo_norm_rows_with(dtype, X, Y, Wt, row0, nrows, bs, dim, BM, BN, rldn, RA, eps, stream_rows, grid < 0,
+                             grid < 0 ? -grid : grid, stream);
 }
 
 extern "C" int fo_rmsnorm(int dtype, const void *X, void *Y, const void *Wt, int bs, int dim,

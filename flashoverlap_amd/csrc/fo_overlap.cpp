@@ -3,6 +3,7 @@
 // streams; every call only enqueues work and returns.  May be captured into a HIP graph.
 #include <mutex>
 #include <new>
+#include <vector>
 
 #include "fo_common.h"
 
@@ -285,11 +286,54 @@ extern "C" int fo_overlap_gemm(fo_overlap_t *h, int dtype, int M, int N, int K, 
 
 namespace {
 
+// The reorder+RMSNorm that follows the overlapped GEMM in the reference's layers (example/RMSNorm.py:20-34
+// behind example/RowParallelLinear.py:50-66), enqueued by the overlapped call itself: a tile row of the output
+// can be normalised as soon as the group that holds its last tile has been consumed, so the rows follow the
+// consumer batch by batch on the consumer stream and only the last batch's rows remain behind the GEMM.
+struct norm_plan {
+    void *Y = nullptr;
+    const void *Wt = nullptr;
+    float eps = 0.f;
+    const int32_t *RA_host = nullptr;
+};
+
+// Rows of tile rows [first, end) of Y, on `stream`.
+int norm_tile_rows(const norm_plan &np, int dtype, const void *C, int M, int N, int BM, int BN, int rLDN,
+                   const int32_t *RA, int first, int end, bool beside_gemm, fo_stream_t stream) {
+    return fo_norm_rows_with(dtype, C, np.Y, np.Wt, first * BM, (end - first) * BM, M, N, BM, BN, rLDN, RA, np.eps,
+                             fo_streams((int64_t)M * N * 4), beside_gemm, 0, stream);
+}
+
+// Tile rows whose tiles all lie in storage slots below `done` and that have not been normalised yet, as
+// runs of consecutive tile rows; at most kMaxRuns launches per batch (a reorder table that scatters the rows
+// of a wave leaves the rest to the last batch).  last_slot[tm] = largest slot of tile row tm; -1 once normalised.
+constexpr int kMaxRuns = 4;
+int norm_ready_rows(const norm_plan &np, long *last_slot, int TM, long done, bool final_batch, int dtype, const void *C,
+                    int M, int N, int BM, int BN, int rLDN, const int32_t *RA, bool beside_gemm, fo_stream_t stream) {
+    int runs = 0;
+    for (int tm = 0; tm < TM;) {
+        if (last_slot[tm] < 0 || last_slot[tm] >= done) {
+            tm++;
+            continue;
+        }
+        int end = tm;
+        while (end < TM && last_slot[end] >= 0 && last_slot[end] < done) end++;
+        if (!final_batch && runs == kMaxRuns) break;
+        int rc = norm_tile_rows(np, dtype, C, M, N, BM, BN, rLDN, RA, tm, end, beside_gemm, stream);
+        if (rc) return rc;
+        for (int t = tm; t < end; t++) last_slot[t] = -1;
+        runs++;
+        tm = end;
+    }
+    return FO_OK;
+}
+
 // GemmAllReduceOverlap on whatever `h` describes: a caller's handle, or the
-// streams and static workspace of a handle-free call.
+// streams and static workspace of a handle-free call.  np: the normalisation to enqueue behind the consumer
+// (null: none).
 int allreduce_overlap(fo_overlap *h, int dtype, int M, int N, int K, const void *A, const void *B, void *C,
                       int32_t *MM, const int32_t *RA, int TM, int TN, int rLDN, const int32_t *cseg_host,
-                      const int32_t *cseg_dev, int G, int algo, int monitor) {
+                      const int32_t *cseg_dev, int G, int algo, int monitor, const norm_plan *np = nullptr) {
     int32_t info[12];
     int rc = fo_algo_info(algo, info);
     if (rc) return rc;
@@ -299,6 +343,18 @@ int allreduce_overlap(fo_overlap *h, int dtype, int M, int N, int K, const void 
     if (rc) return rc;
     const int64_t tile_elems = (int64_t)info[0] * info[1];
     if (h->acc && h->acc_nelem < (int64_t)M * N) return FO_ERR_ARG;
+    std::vector<long> last_slot;  // per tile row: its largest storage slot
+    if (np) {
+        if (!np->Y || !np->Wt || !np->RA_host) return FO_ERR_ARG;
+        if (N % 8 || N > 16384 || (int64_t)M * N * 2 > 0xFFFFFFFFLL) return FO_ERR_SHAPE;
+        last_slot.assign(TM, 0);
+        for (int tm = 0; tm < TM; tm++)
+            for (int tn = 0; tn < TN; tn++) {
+                const long r = np->RA_host[(long)tm * TN + tn];
+                if (r < 0 || r >= (long)TM * TN) return FO_ERR_ARG;
+                if (r > last_slot[tm]) last_slot[tm] = r;
+            }
+    }
 
     const bool same_stream = in_stream(h, M, N, K);
     const int fused = same_stream ? 0 : fused_grid(h, G);
@@ -332,6 +388,10 @@ int allreduce_overlap(fo_overlap *h, int dtype, int M, int N, int K, const void 
                                         h->workspace, fused, fused_slices((int64_t)M * N, G, fused),
                                         fused_poll_gap_ns(M, N, K, fused), stream_acc, h->max_polls, h->comm_stream);
         if (rc) return rc;
+        if (np) {  // that launch ends when the last group has been consumed: every row at once
+            rc = norm_tile_rows(*np, dtype, C, M, N, info[0], info[1], rLDN, RA, 0, TM, false, h->comm_stream);
+            if (rc) return rc;
+        }
     } else {
         int64_t off = 0;
         long done = 0;
@@ -355,6 +415,11 @@ int allreduce_overlap(fo_overlap *h, int dtype, int M, int N, int K, const void 
             }
             off += n;
             done += tiles;
+            if (np) {
+                rc = norm_ready_rows(*np, last_slot.data(), TM, done, j == G, dtype, C, M, N, info[0], info[1], rLDN, RA,
+                                     j < G && !same_stream, cstream);
+                if (rc) return rc;
+            }
             i = j;
         }
     }
@@ -372,6 +437,22 @@ extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int 
     if (!h->gemm_ready || !h->overlap_ready) return FO_ERR_STATE;
     return allreduce_overlap(h, dtype, M, N, K, A, B, C, MM, RA, TM, TN, rLDN, cseg_host, cseg_dev, G, algo,
                              monitor);
+}
+
+extern "C" int fo_overlap_gemm_allreduce_norm(fo_overlap_t *h, int dtype, int M, int N, int K, const void *A,
+                                              const void *B, void *C, int32_t *MM, const int32_t *RA,
+                                              const int32_t *RA_host, int TM, int TN, int rLDN,
+                                              const int32_t *cseg_host, const int32_t *cseg_dev, int G, int algo,
+                                              int monitor, void *Y, const void *Wt, float eps) {
+    if (!h || !MM) return FO_ERR_ARG;
+    if (!h->gemm_ready || !h->overlap_ready) return FO_ERR_STATE;
+    norm_plan np;
+    np.Y = Y;
+    np.Wt = Wt;
+    np.eps = eps;
+    np.RA_host = RA_host;
+    return allreduce_overlap(h, dtype, M, N, K, A, B, C, MM, RA, TM, TN, rLDN, cseg_host, cseg_dev, G, algo, monitor,
+                             &np);
 }
 
 extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, int N, int K,

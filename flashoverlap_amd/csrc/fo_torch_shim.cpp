@@ -128,6 +128,27 @@ struct OverlapImpl : torch::CustomClassHolder {
               "gemm_allreduce_overlap");
     }
 
+    // Addition: gemm_allreduce_overlap followed by reorder_rmsnorm(C -> Y) with the rows normalised on the consumer
+    // stream as the groups that complete them are consumed (fo_overlap_gemm_allreduce_norm); RA_CPU is a host copy of RA.
+    void gemm_allreduce_rmsnorm_overlap(at::Tensor A, at::Tensor B, at::Tensor C, at::Tensor MM, at::Tensor RA,
+                                        at::Tensor RA_CPU, int64_t rLDN, at::Tensor cSEG_CPU, at::Tensor cSEG_GPU,
+                                        int64_t Algo, bool if_monitor, at::Tensor Y, at::Tensor RW, double eps) {
+        Shape s = gemm_shape(A, B, C);
+        check_buffers(s, Algo, MM, RA, rLDN, cSEG_CPU, cSEG_GPU, if_monitor, nullptr, nullptr, 1);
+        TORCH_CHECK(!acc.defined() || acc.numel() >= (int64_t)s.M * s.N, "flashoverlap: the accumulator is smaller than M*N");
+        TORCH_CHECK(RA_CPU.numel() == RA.numel(), "flashoverlap: RA_CPU must be a host copy of RA");
+        TORCH_CHECK(Y.scalar_type() == C.scalar_type() && RW.scalar_type() == C.scalar_type(),
+                    "flashoverlap: C, Y and RW must share one dtype");
+        TORCH_CHECK(Y.numel() == (int64_t)s.M * s.N && RW.numel() >= s.N, "flashoverlap: need Y[M,N] and RW[N]");
+        check(fo_overlap_gemm_allreduce_norm(h, dtype_of(A), s.M, s.N, s.K, dev_ptr(A, "A"), dev_ptr(B, "B"),
+                                             dev_ptr(C, "C"), dev_i32(MM, "MM"), dev_i32(RA, "RA"),
+                                             host_i32(RA_CPU, "RA_CPU"), (int)RA.size(0), (int)RA.size(1), (int)rLDN,
+                                             host_i32(cSEG_CPU, "cSEG_CPU"), dev_i32(cSEG_GPU, "cSEG_GPU"),
+                                             (int)cSEG_GPU.size(0), (int)Algo, if_monitor ? 1 : 0, dev_ptr(Y, "Y"),
+                                             dev_ptr(RW, "RW"), (float)eps),
+              "gemm_allreduce_rmsnorm_overlap");
+    }
+
     void gemm_reducescatter_overlap(at::Tensor A, at::Tensor B, at::Tensor C, at::Tensor D,
                                     at::Tensor MM, at::Tensor RA, at::Tensor RE, int64_t rLDN,
                                     at::Tensor cSEG_CPU, at::Tensor cSEG_GPU, int64_t Algo,
@@ -312,6 +333,7 @@ TORCH_LIBRARY(flashoverlap_class, m) {
         .def("cutlass_gemm", &OverlapImpl::cutlass_gemm)
         .def("gemm_allreduce_overlap", &OverlapImpl::gemm_allreduce_overlap)
         .def("gemm_reducescatter_overlap", &OverlapImpl::gemm_reducescatter_overlap)
+        .def("gemm_allreduce_rmsnorm_overlap", &OverlapImpl::gemm_allreduce_rmsnorm_overlap)  // addition
         .def("nccl_init", &OverlapImpl::nccl_init)
         .def("gemm_allreduce", &OverlapImpl::gemm_allreduce)
         .def("gemm_reducescatter", &OverlapImpl::gemm_reducescatter)

@@ -191,6 +191,22 @@ def reorder_rmsnorm(X, Y, Wt, BM, BN, rldn, RA, eps=1e-5, stream=None):
                                    _stream(stream)), "fo_reorder_rmsnorm")
 
 
+def reorder_rmsnorm_rows(X, Y, Wt, row0, nrows, BM, BN, rldn, RA, eps=1e-5, stream=None):
+    """Rows [row0, row0 + nrows) of reorder_rmsnorm (RA None: of rmsnorm) with the kernel that fits beside a GEMM."""
+    _check_norm(X, Y, Wt)
+    bs, dim = X.shape
+    if row0 < 0 or nrows < 0 or row0 + nrows > bs:
+        raise ValueError(f"rows {row0}..{row0 + nrows - 1} lie outside the {bs} rows of X")
+    if RA is not None:
+        if BM <= 0 or BN <= 0 or bs % BM or dim % BN:
+            raise ValueError(f"[{bs}, {dim}] is not a multiple of the tile {BM} x {BN}")
+        if RA.numel() < (bs // BM) * (dim // BN):
+            raise ValueError(f"RA holds {RA.numel()} entries, the matrix has {(bs // BM) * (dim // BN)} tiles")
+    check(lib().fo_reorder_rmsnorm_rows(dtype_code(X), _ptr(X, "X"), _ptr(Y, "Y"), _ptr(Wt, "W"), int(row0), int(nrows),
+                                        bs, dim, int(BM), int(BN), int(rldn), None if RA is None else _i32(RA, "RA"),
+                                        float(eps), _stream(stream)), "fo_reorder_rmsnorm_rows")
+
+
 def rmsnorm(X, Y, Wt, eps=1e-5, stream=None):
     _check_norm(X, Y, Wt)
     bs, dim = X.shape
@@ -278,6 +294,26 @@ class Overlap:
             _i32(RA, "RA"), TM, TN, int(rLDN), _i32(cseg_cpu, "cSEG_CPU", cuda=False),
             _i32(cseg_gpu, "cSEG_GPU"), cseg_gpu.numel(), int(algo), int(bool(monitor))),
             "fo_overlap_gemm_allreduce")
+
+    def gemm_allreduce_rmsnorm_overlap(self, A, B, C, MM, RA, RA_cpu, rLDN, cseg_cpu, cseg_gpu, algo, Y, Wt,
+                                       eps=1e-5, monitor=False):
+        """gemm_allreduce_overlap + reorder_rmsnorm(C -> Y) in one call: the rows are normalised on the consumer
+        stream as the groups that complete them have been consumed.  RA_cpu: host copy of RA (None: copied here,
+        which synchronises)."""
+        M, N, K = self._check_call(A, B, C, MM, RA, rLDN, cseg_cpu, cseg_gpu, algo, monitor)
+        TM, TN = RA.shape
+        if RA_cpu is None:
+            RA_cpu = RA.cpu()
+        if RA_cpu.is_cuda or RA_cpu.numel() != RA.numel():
+            raise ValueError("RA_cpu must be a host copy of RA")
+        _same_dtype(A, Y, Wt)
+        if Y.numel() != M * N or Wt.numel() < N:
+            raise ValueError("need Y with M*N elements and a weight of N elements")
+        check(lib().fo_overlap_gemm_allreduce_norm(
+            self._h, dtype_code(A), M, N, K, _ptr(A), _ptr(B), _ptr(C), _i32(MM, "MM"), _i32(RA, "RA"),
+            _i32(RA_cpu, "RA_cpu", cuda=False), TM, TN, int(rLDN), _i32(cseg_cpu, "cSEG_CPU", cuda=False),
+            _i32(cseg_gpu, "cSEG_GPU"), cseg_gpu.numel(), int(algo), int(bool(monitor)), _ptr(Y, "Y"),
+            _ptr(Wt, "W"), float(eps)), "fo_overlap_gemm_allreduce_norm")
 
     def gemm_reducescatter_overlap(self, A, B, C, D, MM, RA, RE, rLDN, cseg_cpu, cseg_gpu, algo,
                                    monitor=False):

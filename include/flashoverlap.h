@@ -228,6 +228,16 @@ int fo_wait_reduce_groups(int dtype, const void *C, void *ACC, int32_t *MM,
 int fo_reorder_rmsnorm(int dtype, const void *X, void *Y, const void *Wt, int bs, int dim, int BM,
                        int BN, int rldn, const int32_t *RA, float eps, fo_stream_t stream);
 
+/* Rows [row0, row0 + nrows) of fo_reorder_rmsnorm (RA == NULL: of fo_rmsnorm): the
+ * same arithmetic, src/rmsnorm/rmsnorm.cuh:64-117, for a range of output rows
+ * whose tiles are complete while others are still being computed.  The kernel
+ * is thin enough (registers, LDS) to run beside a GEMM that holds every CU;
+ * fo_overlap_gemm_allreduce_norm enqueues it wave by wave.  bs * dim * 2 bytes
+ * must stay below 4 GiB and dim <= 16384. */
+int fo_reorder_rmsnorm_rows(int dtype, const void *X, void *Y, const void *Wt, int row0, int nrows, int bs,
+                            int dim, int BM, int BN, int rldn, const int32_t *RA, float eps,
+                            fo_stream_t stream);
+
 /* Replaces rmsnorm(X, RX, RW), src/rmsnorm/rmsnorm.cu:32-46, kernel rmsnorm.cuh:14-59. */
 int fo_rmsnorm(int dtype, const void *X, void *Y, const void *Wt, int bs, int dim, float eps,
                fo_stream_t stream);
@@ -300,6 +310,27 @@ int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int N, int K, c
                               const void *B, void *C, int32_t *MM, const int32_t *RA, int TM,
                               int TN, int rLDN, const int32_t *cseg_host,
                               const int32_t *cseg_dev, int G, int algo, int monitor);
+/* fo_overlap_gemm_allreduce followed by fo_reorder_rmsnorm(C -> Y, Wt, eps) over the
+ * same tiles (BM, BN of the Algo, RA, rLDN), as the reference's layers chain them
+ * (example/RowParallelLinear.py:50-66 then example/RMSNorm.py:20-34, kernel
+ * src/rmsnorm/rmsnorm.cuh:64-117), with the normalisation enqueued by the overlapped
+ * call itself; no counterpart in the reference, where it is a separate call that
+ * starts after the join.  A tile row of the output is normalised as soon as the group
+ * holding its last tile has been consumed: behind each wait + consumer batch the
+ * consumer stream gets the rows that batch completed (runs of consecutive tile
+ * rows, at most four launches per batch; what a scattered reorder table leaves over
+ * goes behind the last batch), so with a reorder table built from fo_schedule_order
+ * and whole-row waves (fo_gemm_set_row_waves) only the last wave's consumer and rows
+ * remain behind the GEMM.  RA_host: a host copy of RA (the call plans from it; it is
+ * not kept).  Y[M,N] row-major, Wt[N]; N <= 16384, M*N*2 bytes below 4 GiB.  The GEMM
+ * stream continues when Y is complete.  Results: C, MM and the accumulator exactly as
+ * fo_overlap_gemm_allreduce leaves them; Y as fo_reorder_rmsnorm_rows computes it
+ * (same arithmetic as fo_reorder_rmsnorm, partial sums in another order). */
+int fo_overlap_gemm_allreduce_norm(fo_overlap_t *h, int dtype, int M, int N, int K, const void *A,
+                                   const void *B, void *C, int32_t *MM, const int32_t *RA,
+                                   const int32_t *RA_host, int TM, int TN, int rLDN,
+                                   const int32_t *cseg_host, const int32_t *cseg_dev, int G, int algo,
+                                   int monitor, void *Y, const void *Wt, float eps);
 /* GemmReduceScatterOverlap(...), src/overlap_impl.cu:266-321.  D[M/W, N]
  * receives this rank's chunk of every group at offset acc/W (sum over the one
  * rank present); with an accumulator attached all W chunks are accumulated. */

@@ -38,7 +38,8 @@ def test_shim_registers_reference_names():
     ov = torch.classes.flashoverlap_class.OverlapImpl()
     for m in ["nccl_init", "cutlass_init", "overlap_init", "cutlass_gemm", "gemm_allreduce_overlap",
               "gemm_reducescatter_overlap", "gemm_allreduce", "gemm_reducescatter", "gemm_all2all",
-              "nccl_allreduce", "nccl_reducescatter", "nccl_all2all", "seg_allreduce"]:
+              "nccl_allreduce", "nccl_reducescatter", "nccl_all2all", "seg_allreduce",
+              "gemm_allreduce_rmsnorm_overlap"]:     # the last one is an addition
         assert hasattr(ov, m), m
     bl = torch.classes.flashoverlap_class.BaselineImpl()
     for m in ["nccl_init", "cublas_init", "cublas_gemm", "gemm_allreduce", "gemm_reducescatter",
