@@ -111,6 +111,8 @@ int fo_gemm_reordered_quiet(int dtype, int M, int N, int K, int rLDN, const int3
 // that it is left cacheable, because the next kernel reads it again.
 constexpr int64_t kStreamAboveBytes = 192LL << 20;
 inline bool fo_streams(int64_t bytes) { return bytes > kStreamAboveBytes; }
+// A GEMM output above this size is stored with the non-temporal hint (see store16_nt in fo_gemm_kernel.h).
+constexpr int64_t kStreamOutAboveBytes = 96LL << 20;
 
 // The consumer entry points with the accumulator's cache policy chosen by the
 // caller (fo_aux.hip; the extern "C" forms decide from their own range).

@@ -90,6 +90,7 @@ int run_gemm(int mode, int dtype, int M, int N, int K, int rLDN, const int32_t *
     a.first = 0; a.sub_m = a.sub_n = 1;
     a.count = r.grid_m * r.grid_n - r.tail_tiles;
     a.quiet = quiet ? 1 : 0;
+    a.stream_out = (int64_t)M * N * 2 > kStreamOutAboveBytes ? 1 : 0;
     if (mode != MODE_PLAIN) {
         const long T = (long)(M / a.BM) * a.TN;
         if ((!MM && !quiet) || !RA || !cseg) return FO_ERR_ARG;

@@ -233,20 +233,37 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
     for (int q = 0; q < NPRE; q++) pre[q] = 0;
     const bool reg_search = p.G <= kPrefixRegs;
     const bool signalling = MODE != MODE_PLAIN && !p.quiet;
+    // The group sizes are requested in front of the pipeline fill and summed behind it (a round trip to memory and
+    // some two dozen dependent cross-lane steps otherwise stand between the kernel's start and its first operand
+    // load).  The requests are assembly: their registers are read only behind the fill's wait for loads that were
+    // requested after them, and the compiler, which knows nothing of the fill's loads, would otherwise wait for
+    // every one of those as well.  Lanes beyond G ask for element 0.
+    int cs_raw[NPRE];
     if (signalling && reg_search) {
-        int base = 0;
 #pragma unroll
         for (int q = 0; q < NPRE; q++) {
-            int v = q * 64 + lane < p.G ? p.cseg[q * 64 + lane] : 0;
-#pragma unroll
-            for (int d = 1; d < 64; d <<= 1) {
-                int o = __shfl_up(v, d, 64);
-                if (lane >= d) v += o;
-            }
-            pre[q] = v + base;
-            base = __shfl(pre[q], 63, 64);
+            const int32_t *src = p.cseg + (q * 64 + lane < p.G ? q * 64 + lane : 0);
+            asm volatile("global_load_dword %0, %1, off" : "=v"(cs_raw[q]) : "v"(src) : "memory");
         }
     }
+    auto sum_groups = [&]() {
+        if (signalling && reg_search) {
+            int base = 0;
+#pragma unroll
+            for (int q = 0; q < NPRE; q++) {
+                if (q * 64 < p.G) {  // wave-uniform
+                    int v = q * 64 + lane < p.G ? cs_raw[q] : 0;
+#pragma unroll
+                    for (int d = 1; d < 64; d <<= 1) {
+                        int o = __shfl_up(v, d, 64);
+                        if (lane >= d) v += o;
+                    }
+                    pre[q] = v + base;
+                    base = __shfl(pre[q], 63, 64);
+                }
+            }
+        }
+    };
     auto group_of = [&](int r) {
         if (reg_search) {
 #pragma unroll
@@ -258,32 +275,30 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
         }
         return find_group(p.cseg, p.G, r, lane);
     };
-    // Wavefront 0 announces the reorder tiles at slots rs[] with groups gs[].  Callers guarantee that every
-    // wavefront's write-through stores of those tiles are acknowledged (vmcnt) and that a workgroup barrier
-    // lies between that wait and this call, so the atomic itself is relaxed.
+    // Wavefront 0 announces a macro tile's reorder tiles: lane s < nsub holds the storage slot r and the group g of
+    // reorder tile s (one register each; as scalars, slots and groups of this tile and of the one whose signal is
+    // still owed took twenty scalar registers through the K loop and the kernel spilled 145 of them).  Callers
+    // guarantee that every wavefront's write-through stores of those tiles are acknowledged (vmcnt) and that a
+    // workgroup barrier lies between that wait and this call, so the atomic itself is relaxed.
     // Reorder tiles of one group are counted with one atomic: all resident workgroups finish a tile at about the
     // same time and bump the same few counters, and atomics on one address complete one after the other, some 25 ns
     // apart (512 tiles of 256x256 in 128x128 reorder tiles, 8 groups: 7 us per launch with one atomic per tile).
-    auto announce = [&](const int (&rs)[kMaxSub], const int (&gs)[kMaxSub]) {
+    auto announce = [&](int r, int g) {
+        int count = 0;      // tiles of this lane's group from this lane on
+        bool first = true;  // no earlier tile of this group
 #pragma unroll
-        for (int s = 0; s < kMaxSub; s++) {
-            if (s < nsub) {
-                const int r = rs[s];
-                const int g = gs[s];
-                int count = 1;       // tiles s, s+1, ... of this group
-                bool first = true;   // no earlier tile of this group
-#pragma unroll
-                for (int q = 0; q < kMaxSub; q++) {
-                    if (q < s && gs[q] == g) first = false;
-                    if (q > s && q < nsub && gs[q] == g) count++;
-                }
-                if (lane == 0) {
-                    if (first) __hip_atomic_fetch_add(p.MM + g, count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    if (p.monitor) {
-                        int o = __hip_atomic_fetch_add(p.MM + (p.TN - 1), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        __hip_atomic_store(p.MM + p.TN + r, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    }
-                }
+        for (int q = 0; q < kMaxSub; q++) {
+            const int gq = __builtin_amdgcn_readlane(g, q);
+            if (q < nsub && gq == g) {
+                if (q < lane) first = false;
+                if (q >= lane) count++;
+            }
+        }
+        if (lane < nsub) {
+            if (first) __hip_atomic_fetch_add(p.MM + g, count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (p.monitor) {
+                int o = __hip_atomic_fetch_add(p.MM + (p.TN - 1), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(p.MM + p.TN + r, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
     };
@@ -303,9 +318,23 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
                 if (s < nsub) rs_next[s] = RAc[(tm_ * (MT / p.BM) + s / sub_n) * p.TN + tn_ * sub_n + s % sub_n];
         }
     };
-    int prev_rs[kMaxSub] = {0, 0, 0, 0};  // slots and groups of the tile whose signal is still owed
-    int prev_gs[kMaxSub] = {0, 0, 0, 0};
-    int owed = 0;          // PUB meetings until that signal may be sent
+    // The slots that request_slots brought, as the rest of the kernel uses them: this wavefront's own reorder tile as a
+    // scalar, all of them in lanes 0 .. nsub-1 of one register.
+    const int my_sub = __builtin_amdgcn_readfirstlane(((wm * 128) / p.BM) * sub_n + (wn * 128) / p.BN);
+    int r_mine = 0, v_rs = 0;
+    auto take_slots = [&]() {
+        if (MODE != MODE_PLAIN) {
+#pragma unroll
+            for (int s = 0; s < kMaxSub; s++) {
+                int rr = rs_next[s];
+                asm volatile("" : "+s"(rr));  // the scalar loads complete here
+                if (s == my_sub) r_mine = rr;
+                v_rs = lane == s ? rr : v_rs;
+            }
+        }
+    };
+    int v_prev_r = 0, v_prev_g = 0;  // slots and groups (per lane) of the tile whose signal is still owed
+    int owed = 0;                    // PUB meetings until that signal may be sent
 
     fo_float4v acc[F][F];
     fo_u32x4 af[ARING], bf[2][F];
@@ -331,6 +360,7 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
     for (int j = 0; j < F; j++) load_b(0, lb0, 0, j);
 #pragma unroll
     for (int i = 0; i < AHEAD; i++) load_a(i, la0, 0, i);
+    sum_groups();  // the group sizes arrived before stage 0 did (requested earlier, vmcnt retires in issue order)
 
     int tile = blockIdx.x;
     unsigned slot_b = 0;  // byte offset of the slot the next K step reads
@@ -339,22 +369,13 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
         fo_unit_to_tile(tile, p.first, p.sub_m, p.sub_n, p.grid_m, p.grid_n, p.panel, p.xcd_remap, &pm, &pn);
         pm = __builtin_amdgcn_readfirstlane(pm);
         pn = __builtin_amdgcn_readfirstlane(pn);
-        int rs[kMaxSub] = {0, 0, 0, 0};  // storage slots of this macro tile's reorder tiles
-        if (MODE != MODE_PLAIN) {
-#pragma unroll
-            for (int s = 0; s < kMaxSub; s++) {
-                rs[s] = rs_next[s];
-                asm volatile("" : "+s"(rs[s]));  // the scalar loads complete here
-            }
-        }
+        if (tile == (int)blockIdx.x) take_slots();  // later tiles: taken inside the previous tile's epilogue
         // Scatter: the row map entries of the wavefront's 128 rows, two per lane (lane l: rows l and 64 + l), are
         // requested here and rest in two registers through the K loop; the epilogue hands them to the lanes that
         // store each row.  Requested in the epilogue they cost every tile a round trip to memory with nothing to hide it.
         int32_t re_lo = 0, re_hi = 0;
         if (MODE == MODE_SCATTER) {
-            const int s = ((wm * 128) / p.BM) * sub_n + (wn * 128) / p.BN;
-            const int r = s == 0 ? rs[0] : s == 1 ? rs[1] : s == 2 ? rs[2] : rs[3];
-            const long trow = (long)(r / p.rLDN) * p.BM + (wm * 128) % p.BM;
+            const long trow = (long)(r_mine / p.rLDN) * p.BM + (wm * 128) % p.BM;
             re_lo = p.RE[trow + lane];
             re_hi = p.RE[trow + 64 + lane];
         }
@@ -366,7 +387,14 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
                 for (int v = 0; v < 4; v++) acc[i][j][v] = 0.f;
         fo_mfma_fence();
 
+        // A tile whose predecessor's signal is still owed leaves the K loop after its first step, sends the signal and
+        // re-enters: that step's PUB meeting has waited for the predecessor's stores in every wavefront (part of the
+        // stage's loads was requested behind them, rows 0-5, and vmcnt retires in issue order), with the meeting's
+        // barrier behind the wait.  The test inside the step (one scalar compare and branch per K step, after the PUB
+        // meeting) cost the large square 4 us.
         int kt = 0;
+        int kt_stop = (MODE != MODE_PLAIN && owed > 0) ? 1 : KT;
+        for (;;) {
         do {
             unsigned la_ = la0 ^ slot_b, lb_ = lb0 ^ slot_b;
             asm volatile("" : "+v"(la_), "+v"(lb_));
@@ -442,27 +470,27 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
                     wait_vmcnt<YOUNG>();
                     __builtin_amdgcn_s_barrier();
                     asm volatile("" ::: "memory");
-                    if (MODE != MODE_PLAIN) {
-                        if (owed > 0) {
-                            if (--owed == 0) {
-                                if (wave == 0) announce(prev_rs, prev_gs);
-                                // Nothing scalar stays in flight behind this rare path: with a scalar load possibly
-                                // pending, the K loop's waits for LDS data would all have to be waits for everything.
-                                __builtin_amdgcn_s_waitcnt(0xC07F);
-                            }
-                        }
-                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
             slot_b ^= SLOT_B;
-        } while (++kt < KT);
+        } while (++kt < kt_stop);
+            if (MODE == MODE_PLAIN || owed == 0) break;
+            owed = 0;
+            if (wave == 0) announce(v_prev_r, v_prev_g);
+            // Nothing scalar stays in flight behind this rare path: with a scalar load possibly pending, the K
+            // loop's waits for LDS data would all have to be waits for everything.
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            if (kt >= KT) break;
+            kt_stop = KT;
+        }
 
         fo_mfma_fence();
         const int next = tile + gridDim.x;
         const bool has_next = next < ntiles;
         if (has_next) request_slots(next);
 
+        int v_done = 0;  // the slots of the tile that this epilogue stores (per lane)
         // ---- epilogue.  A wavefront's 128x128 block lies inside one reorder tile (BM and BN are multiples of
         // 128), so slot and base address are scalars.  The lane id is laundered so that this addressing is
         // recomputed per tile instead of living in registers across the K loop.
@@ -474,15 +502,13 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
             const int srow = el / CPR, scol = el % CPR;
             const int ldp = MODE == MODE_PLAIN ? p.N : p.rLDN * p.BN;  // leading dimension of the output view
             const int row0 = (wm * 128) % p.BM, col0 = (wn * 128) % p.BN;
-            int r = 0;
-            if (MODE != MODE_PLAIN) {
-                const int s = ((wm * 128) / p.BM) * sub_n + (wn * 128) / p.BN;
-                r = s == 0 ? rs[0] : s == 1 ? rs[1] : s == 2 ? rs[2] : rs[3];
-            }
+            const int r = r_mine;
+            const int v_cur = v_rs;  // this tile's slots: the next tile's replace them inside the loop below
             const long trow = MODE == MODE_PLAIN ? (long)pm * MT + wm * 128 : (long)(r / p.rLDN) * p.BM + row0;
             const long tcol = MODE == MODE_PLAIN ? (long)pn * MT + wn * 128 : (long)(r % p.rLDN) * p.BN + col0;
             char *cbase = reinterpret_cast<char *>(p.C) + (trow * ldp + tcol) * 2;  // wave-uniform
             const unsigned lane_off = (unsigned)(srow * ldp + scol * 8) * 2;
+            const bool stream_out = p.stream_out != 0;  // wave-uniform
 #pragma unroll
             for (int i = 0; i < F; i++) {  // 16 output rows = one row of accumulator blocks
                 __builtin_amdgcn_sched_barrier(0);
@@ -511,33 +537,49 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
                         // row i * 16 + ps * RPP + srow of the block: its entry sits in that lane of re_lo / re_hi
                         const long prow = __builtin_amdgcn_ds_bpermute(((i * 16 + ps * RPP) % 64 + srow) * 4,
                                                                        i * 16 + ps * RPP < 64 ? re_lo : re_hi);
-                        store16_write_through(p.C + (size_t)prow * ldp + tcol + scol * 8, v);
+                        if (stream_out)
+                            store16_write_through_nt(p.C + (size_t)prow * ldp + tcol + scol * 8, v);
+                        else
+                            store16_write_through(p.C + (size_t)prow * ldp + tcol + scol * 8, v);
                     } else {
                         char *sb = cbase + (size_t)(i * 16 + ps * RPP) * ldp * 2;
-                        if (MODE == MODE_PLAIN)
-                            store16(sb, lane_off, v);
-                        else
-                            store16_write_through(sb, lane_off, v);
+                        if (MODE == MODE_PLAIN) {
+                            if (stream_out)
+                                store16_nt(sb, lane_off, v);
+                            else
+                                store16(sb, lane_off, v);
+                        } else {
+                            if (stream_out)
+                                store16_write_through_nt(sb, lane_off, v);
+                            else
+                                store16_write_through(sb, lane_off, v);
+                        }
                     }
                 }
                 __builtin_amdgcn_s_waitcnt(0xC07F);  // strip reads done before the next pass overwrites it
                 __builtin_amdgcn_wave_barrier();
+                // The next tile's slots, requested in front of this epilogue, have arrived with the pass's waits: they
+                // leave their four scalar registers here.
+                if (i == 0 && has_next) take_slots();
             }
+            v_done = v_cur;
         }
 
         if (signalling) {
-            int gs[kMaxSub] = {0, 0, 0, 0};
+            int v_g = 0;  // lane s: group of reorder tile s
             if (wave == 0) {
 #pragma unroll
-                for (int s = 0; s < kMaxSub; s++) gs[s] = s < nsub ? group_of(rs[s]) : 0;
+                for (int s = 0; s < kMaxSub; s++) {
+                    if (s < nsub) {
+                        const int g = group_of(__builtin_amdgcn_readlane(v_done, s));
+                        v_g = lane == s ? g : v_g;
+                    }
+                }
             }
             if (has_next) {
                 owed = 1;  // PUB meetings until this tile's stores have been waited for in every wavefront
-#pragma unroll
-                for (int s = 0; s < kMaxSub; s++) {
-                    prev_rs[s] = rs[s];
-                    prev_gs[s] = gs[s];
-                }
+                v_prev_r = v_done;
+                v_prev_g = v_g;
             } else {
                 // Last tile: every lane waits until its own write-through stores are acknowledged, the barrier
                 // collects the workgroup, then one lane bumps the counters (the reference has no fence here,
@@ -546,8 +588,8 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
                 __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
                 if (wave == 0) {
-                    if (owed > 0) announce(prev_rs, prev_gs);
-                    announce(rs, gs);
+                    if (owed > 0) announce(v_prev_r, v_prev_g);
+                    announce(v_done, v_g);
                 }
             }
         }
