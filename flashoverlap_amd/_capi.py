@@ -42,6 +42,7 @@ SIGNATURES = {
                                    vp]),
     "fo_reorder_rmsnorm_rows": (c_int, [c_int, vp, vp, vp, c_int, c_int, c_int, c_int, c_int, c_int, c_int, vp, c_f32,
                                         vp]),
+    "fo_norm_rows_kernel_info": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, vp]),
     "fo_rmsnorm": (c_int, [c_int, vp, vp, vp, c_int, c_int, c_f32, vp]),
     "fo_overlap_plan_batches": (c_int, [vp, c_int, c_int, vp]),
     "fo_overlap_create": (c_int, [ctypes.POINTER(vp)]),
@@ -164,6 +165,14 @@ def kernel_info(algo, M, N, epilogue=1, dtype=F16):
     info = (ctypes.c_int32 * 4)()
     check(lib().fo_gemm_kernel_info(int(dtype), int(algo), M, N, int(epilogue), info), "fo_gemm_kernel_info")
     return {"resident": info[0], "vgprs": info[1], "lds_bytes": info[2], "threads": info[3]}
+
+
+def norm_rows_kernel_info(dim, reorder=True, BN=128, rldn=1, beside_gemm=True, dtype=F16):
+    """{vector registers per lane, LDS bytes per workgroup} of the row-range RMSNorm kernel; asks the GPU."""
+    info = (ctypes.c_int32 * 2)()
+    check(lib().fo_norm_rows_kernel_info(int(dtype), int(dim), int(bool(reorder)), int(BN), int(rldn),
+                                         int(bool(beside_gemm)), info), "fo_norm_rows_kernel_info")
+    return {"vgprs": info[0], "lds_bytes": info[1]}
 
 
 def plan_batches(cseg, wave_tiles):

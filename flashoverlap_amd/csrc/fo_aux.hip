@@ -534,6 +534,13 @@ int launch_rmsnorm_as(const void *X, void *Y, const void *Wt, int bs, int dim, i
 template <typename Tag>
 int launch_rmsnorm(const void *X, void *Y, const void *Wt, int bs, int dim, int BM, int BN,
                    int rldn, const int32_t *RA, float eps, hipStream_t stream) {
+    // Rows of exactly 8192 elements fill the row kernel's workgroup (four wavefronts per row, four chunks per
+    // lane), and there it is the faster of the two: 8192 x 8192, nothing cached, 45.5-46.7 us against 47-50
+    // (fp16 and bf16, reorder or not).  Narrower rows leave its lanes idle (16384 x 1024: 15.5 against 11.8 us)
+    // and longer ones cost it its look-ahead.
+    if (dim == 8192 && (int64_t)bs * dim * 2 <= 0xFFFFFFFFLL)
+        return fo_norm_rows_with(std::is_same<Tag, fo_bf16_tag>::value ? FO_BF16 : FO_F16, X, Y, Wt, 0, bs, bs, dim, BM,
+                                 BN, rldn, RA, eps, fo_streams((int64_t)bs * dim * 4), false, 0, stream);
     // input and output together against the cache that would have to hold them
     if (fo_streams((int64_t)bs * dim * 4))
         return launch_rmsnorm_as<Tag, true>(X, Y, Wt, bs, dim, BM, BN, rldn, RA, eps, stream);
@@ -556,7 +563,7 @@ int launch_rmsnorm(const void *X, void *Y, const void *Wt, int bs, int dim, int 
 // 512 (at most 408 with the accumulators); rows above 8192 elements (CH = 8) do without the look-ahead
 // and may take 128, which fits beside the plain GEMM's wavefront only.
 template <typename Tag, int CH, bool STREAM, int PATH>
-__global__ __launch_bounds__(256, CH <= 4 ? 5 : 4) void fo_norm_rows_kernel(const fo_u32x4 *X, fo_u32x4 *Y, const fo_u32x4 *Wt,
+__global__ __launch_bounds__(256, (CH <= 4 && !(CH == 4 && std::is_same<Tag, fo_bf16_tag>::value)) ? 5 : 4) void fo_norm_rows_kernel(const fo_u32x4 *X, fo_u32x4 *Y, const fo_u32x4 *Wt,
                                                               int row0, int nrows, int rows_per_wg, int dim, int BM,
                                                               int BN, int rldn, const int32_t *RA, float eps,
                                                               unsigned x_bytes) {
@@ -692,8 +699,10 @@ __global__ __launch_bounds__(256, CH <= 4 ? 5 : 4) void fo_norm_rows_kernel(cons
 // kBesideGemmLds bytes of LDS it never touches (one workgroup per CU beside the GEMM's, as for the consumer).
 template <typename Tag, bool STREAM, int PATH>
 int launch_norm_rows_on(const void *X, void *Y, const void *Wt, int row0, int nrows, int dim, int BM, int BN, int rldn,
-                        const int32_t *RA, float eps, bool beside_gemm, int grid, unsigned x_bytes, hipStream_t stream) {
+                        const int32_t *RA, float eps, bool beside_gemm, int grid, unsigned x_bytes, hipStream_t stream,
+                        int32_t *info) {
     const int nch = dim / 8;
+    if (nrows < 1) nrows = 1;  // the query for the kernel's resources comes with no rows
     if (grid <= 0) grid = (nrows + 1) / 2;
     const int most = beside_gemm ? 256 : 4096;
     if (grid > most) grid = most;
@@ -703,19 +712,28 @@ int launch_norm_rows_on(const void *X, void *Y, const void *Wt, int row0, int nr
     const fo_u32x4 *x = static_cast<const fo_u32x4 *>(X);
     fo_u32x4 *y = static_cast<fo_u32x4 *>(Y);
     const fo_u32x4 *w = static_cast<const fo_u32x4 *>(Wt);
-#define FO_NORM_ROWS(CH_)                                                                                          \
+    // info != null: nothing is launched; info = {registers per lane, LDS bytes per workgroup} of the kernel that would run
+#define FO_NORM_ROWS(CH_)                                                                                               \
+    if (info) {                                                                                                         \
+        hipFuncAttributes attr;                                                                                         \
+        FO_HIP_CHECK(hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(&fo_norm_rows_kernel<Tag, CH_, STREAM, PATH>))); \
+        info[0] = attr.numRegs;                                                                                         \
+        info[1] = (int)attr.sharedSizeBytes + lds;                                                                      \
+        return FO_OK;                                                                                                   \
+    }                                                                                                                   \
     hipLaunchKernelGGL((fo_norm_rows_kernel<Tag, CH_, STREAM, PATH>), dim3(grid), dim3(256), lds, stream, x, y, w, row0, \
                        nrows, rows_per_wg, dim, BM, BN, rldn, RA, eps, x_bytes)
-    if (nch <= 256)
+    if (nch <= 256) {
         FO_NORM_ROWS(1);
-    else if (nch <= 512)
+    } else if (nch <= 512) {
         FO_NORM_ROWS(2);
-    else if (nch <= 1024)
+    } else if (nch <= 1024) {
         FO_NORM_ROWS(4);
-    else if (nch <= 2048)
+    } else if (nch <= 2048) {
         FO_NORM_ROWS(8);
-    else
+    } else {
         return FO_ERR_SHAPE;
+    }
 #undef FO_NORM_ROWS
     FO_LAUNCH_CHECK();
     return FO_OK;
@@ -723,15 +741,16 @@ int launch_norm_rows_on(const void *X, void *Y, const void *Wt, int row0, int nr
 
 template <typename Tag, bool STREAM>
 int launch_norm_rows_as(const void *X, void *Y, const void *Wt, int row0, int nrows, int dim, int BM, int BN, int rldn,
-                        const int32_t *RA, float eps, bool beside_gemm, int grid, unsigned x_bytes, hipStream_t stream) {
+                        const int32_t *RA, float eps, bool beside_gemm, int grid, unsigned x_bytes, hipStream_t stream,
+                        int32_t *info) {
     if (!RA)
         return launch_norm_rows_on<Tag, STREAM, NORM_PLAIN>(X, Y, Wt, row0, nrows, dim, BM, BN, rldn, RA, eps, beside_gemm,
-                                                            grid, x_bytes, stream);
+                                                            grid, x_bytes, stream, info);
     if (rldn == 1 && (BN & (BN - 1)) == 0)
         return launch_norm_rows_on<Tag, STREAM, NORM_SLOTS>(X, Y, Wt, row0, nrows, dim, BM, BN, rldn, RA, eps, beside_gemm,
-                                                            grid, x_bytes, stream);
+                                                            grid, x_bytes, stream, info);
     return launch_norm_rows_on<Tag, STREAM, NORM_GENERAL>(X, Y, Wt, row0, nrows, dim, BM, BN, rldn, RA, eps, beside_gemm,
-                                                          grid, x_bytes, stream);
+                                                          grid, x_bytes, stream, info);
 }
 
 // FO_WAIT_MAX_POLLS (environment, read once): bound for the otherwise unbounded
@@ -966,8 +985,8 @@ extern "C" int fo_reorder_rmsnorm(int dtype, const void *X, void *Y, const void 
 
 int fo_norm_rows_with(int dtype, const void *X, void *Y, const void *Wt, int row0, int nrows, int bs, int dim, int BM,
                       int BN, int rldn, const int32_t *RA, float eps, bool stream_rows, bool beside_gemm, int grid,
-                      fo_stream_t stream) {
-    if (!X || !Y || !Wt || bs <= 0 || dim <= 0 || BM <= 0 || BN <= 0 || rldn <= 0) return FO_ERR_ARG;
+                      fo_stream_t stream, int32_t *info) {
+    if (((!X || !Y || !Wt) && !info) || bs <= 0 || dim <= 0 || BM <= 0 || BN <= 0 || rldn <= 0) return FO_ERR_ARG;
     if (row0 < 0 || nrows < 0 || row0 + nrows > bs) return FO_ERR_ARG;
     if (dim % 8 || dim > 16384) return FO_ERR_SHAPE;
     if (RA) {
@@ -975,16 +994,25 @@ int fo_norm_rows_with(int dtype, const void *X, void *Y, const void *Wt, int row
         if (((long)(bs / BM) * (dim / BN)) % rldn) return FO_ERR_SHAPE;
     }
     if ((int64_t)bs * dim * 2 > 0xFFFFFFFFLL) return FO_ERR_SHAPE;  // 32-bit byte offsets into X
-    if (nrows == 0) return FO_OK;
+    if (nrows == 0 && !info) return FO_OK;
     const unsigned x_bytes = (unsigned)((int64_t)bs * dim * 2);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == FO_F16)
-        return stream_rows ? launch_norm_rows_as<fo_f16_tag, true>(X, Y, Wt, row0, nrows, dim, BM, BN, rldn, RA, eps, beside_gemm, grid, x_bytes, s)
-                           : launch_norm_rows_as<fo_f16_tag, false>(X, Y, Wt, row0, nrows, dim, BM, BN, rldn, RA, eps, beside_gemm, grid, x_bytes, s);
+        return stream_rows ? launch_norm_rows_as<fo_f16_tag, true>(X, Y, Wt, row0, nrows, dim, BM, BN, rldn, RA, eps, beside_gemm, grid, x_bytes, s, info)
+                           : launch_norm_rows_as<fo_f16_tag, false>(X, Y, Wt, row0, nrows, dim, BM, BN, rldn, RA, eps, beside_gemm, grid, x_bytes, s, info);
     if (dtype == FO_BF16)
-        return stream_rows ? launch_norm_rows_as<fo_bf16_tag, true>(X, Y, Wt, row0, nrows, dim, BM, BN, rldn, RA, eps, beside_gemm, grid, x_bytes, s)
-                           : launch_norm_rows_as<fo_bf16_tag, false>(X, Y, Wt, row0, nrows, dim, BM, BN, rldn, RA, eps, beside_gemm, grid, x_bytes, s);
+        return stream_rows ? launch_norm_rows_as<fo_bf16_tag, true>(X, Y, Wt, row0, nrows, dim, BM, BN, rldn, RA, eps, beside_gemm, grid, x_bytes, s, info)
+                           : launch_norm_rows_as<fo_bf16_tag, false>(X, Y, Wt, row0, nrows, dim, BM, BN, rldn, RA, eps, beside_gemm, grid, x_bytes, s, info);
     return FO_ERR_DTYPE;
+}
+
+extern "C" int fo_norm_rows_kernel_info(int dtype, int dim, int reorder, int BN, int rldn, int beside_gemm,
+                                        int32_t info[2]) {
+    if (!info || dim <= 0 || dim % 8 || dim > 16384) return FO_ERR_ARG;
+    static const int32_t one = 0;
+    return fo_norm_rows_with(dtype, nullptr, nullptr, nullptr, 0, 0, reorder ? BN : 1, dim, reorder ? BN : 1,
+                             reorder ? BN : 8, reorder ? rldn : 1, reorder ? &one : nullptr, 0.f, true, beside_gemm != 0, 0,
+                             nullptr, info);
 }
 
 extern "C" int fo_reorder_rmsnorm_rows(int dtype, const void *X, void *Y, const void *Wt, int row0, int nrows, int bs,

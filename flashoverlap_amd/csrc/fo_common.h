@@ -141,10 +141,11 @@ int fo_wait_reduce_groups_with(int dtype, const void *C, void *ACC, int32_t *MM,
 
 // Rows [row0, row0 + nrows) of (reorder+)RMSNorm over X[bs, dim] (RA null: no reorder) with the row
 // kernel that fits beside a GEMM (fo_aux.hip).  stream_rows: non-temporal accesses; beside_gemm: at most
-// one workgroup per CU; grid: workgroups (0: chosen from the row count).
+// one workgroup per CU; grid: workgroups (0: chosen from the row count).  info != null: nothing is launched,
+// info = {registers per lane, LDS bytes per workgroup} of the kernel that would run.
 int fo_norm_rows_with(int dtype, const void *X, void *Y, const void *Wt, int row0, int nrows, int bs, int dim, int BM,
                       int BN, int rldn, const int32_t *RA, float eps, bool stream_rows, bool beside_gemm, int grid,
-                      fo_stream_t stream);
+                      fo_stream_t stream, int32_t *info = nullptr);
 
 // The waits with their bound and status word chosen by the caller (fo_aux.hip).
 // max_polls < 0: the bound of the environment variable FO_WAIT_MAX_POLLS (none

@@ -238,6 +238,16 @@ int fo_reorder_rmsnorm_rows(int dtype, const void *X, void *Y, const void *Wt, i
                             int dim, int BM, int BN, int rldn, const int32_t *RA, float eps,
                             fo_stream_t stream);
 
+/* What the kernel behind fo_reorder_rmsnorm_rows occupies (needs a GPU; no counterpart
+ * in the reference): info = {vector registers per lane, LDS bytes per workgroup} of
+ * the variant for rows of dim elements, with a reorder table of BN-wide tiles
+ * (reorder != 0) or without, as launched beside a GEMM (beside_gemm != 0) or alone.
+ * One workgroup of four wavefronts, one per SIMD: it runs beside the signalling
+ * GEMM only while these registers (in eights) and fo_gemm_kernel_info's fit a SIMD's
+ * 512 together, and this LDS fits beside the GEMM workgroup's in the CU's 160 KB. */
+int fo_norm_rows_kernel_info(int dtype, int dim, int reorder, int BN, int rldn, int beside_gemm,
+                             int32_t info[2]);
+
 /* Replaces rmsnorm(X, RX, RW), src/rmsnorm/rmsnorm.cu:32-46, kernel rmsnorm.cuh:14-59. */
 int fo_rmsnorm(int dtype, const void *X, void *Y, const void *Wt, int bs, int dim, float eps,
                fo_stream_t stream);

@@ -157,6 +157,20 @@ def test_row_ranges_of_the_normalisation(fo, oracle, dtype):
         assert ulp_diff_ok(bits_of(Y), bits_of(Y_old), dtype, max_ulp=2, frac=0.99)
 
 
+@pytest.mark.parametrize("dtype,M,N,bm,bn", [(F16, 8192, 8192, 128, 256), (BF16, 8192, 8192, 256, 128),
+                                             (F16, 8192, 4096, 128, 128), (BF16, 4096, 2048, 128, 128)])
+def test_row_kernel_fits_beside_the_signalling_gemm(fo, dtype, M, N, bm, bn):
+    """The rows of a wave are normalised while the next wave's workgroups hold every CU: one workgroup of the row
+    kernel (a wavefront per SIMD) must fit into what a GEMM workgroup leaves of the CU's registers and LDS, or the
+    call silently degrades into GEMM first, normalisation afterwards."""
+    algo = fo._capi.find_algo(bm, bn, swizzle=4)
+    gemm = fo._capi.kernel_info(algo, M, N, epilogue=1, dtype=dtype)
+    rows = fo._capi.norm_rows_kernel_info(N, True, bn, 1, True, dtype=dtype)
+    per_simd = gemm["threads"] // 256 * (gemm["resident"] // 256)
+    assert per_simd * ((gemm["vgprs"] + 7) // 8 * 8) + (rows["vgprs"] + 7) // 8 * 8 <= 512, (gemm, rows)
+    assert (gemm["resident"] // 256) * gemm["lds_bytes"] + rows["lds_bytes"] <= 160 * 1024, (gemm, rows)
+
+
 def test_norm_overlap_refuses_bad_arguments(fo):
     bm, bn, M, N, K = 128, 128, 512, 512, 64
     algo, RA, A, B, gamma, MM, cs_cpu, cs_gpu = _setup(fo, F16, bm, bn, M, N, K, [8, 8], seed=440)
