@@ -111,6 +111,12 @@ __global__ __launch_bounds__(256) void fo_gemm256_kernel(GemmArgs p) {
     constexpr int YOUNG = loads_before_row256(PUB - FREE);       // loads of a step already requested at its PUB meeting
     static_assert(loads_before_row256(kLoadSpan256) == 16, "a stage is sixteen loads per wavefront");
     static_assert(FREE + kLoadSpan256 - ROWS < FREE && PUB > FREE && PUB <= 13, "load rows lie between two FREE meetings");
+    // YOUNG is exact: between a FREE meeting (row 9) and the PUB meeting of the same step (row 12) rows 10-12 issue
+    // loads_in_row256(0..2) loads and nothing else that counts in vmcnt; a tile's stores and the loads of rows 0-5 of
+    // its successor's first step are older than those.  Further vector-memory instructions in that stretch would
+    // only make the PUB wait stricter.  The wait relies on vmcnt retiring loads and stores in issue order (one
+    // counter for both on this part); a part with a counter of its own for stores needs a wait on that one as well.
+    static_assert(YOUNG == loads_in_row256(0) + loads_in_row256(1) + loads_in_row256(2), "loads of rows 10-12");
     static_assert(NST + 16 + YOUNG < 64, "vmcnt range: a tile's stores and a stage's loads in flight together");
     static_assert(FREE + kLoadSpan256 >= ROWS, "the rest of a stage's loads leaves in the rows of the next step");
 
