@@ -228,7 +228,10 @@ def measure(args, workload, compact=False):
         print(json.dumps({"steps_only": True, "steps": K_, "warmup": W_, "ms_per_step": ms}))
         return
     if args.kernels_only and not compact:
-        for fn in (gemm_alone, gemm_signal_alone, consumer_alone, norm):
+        fns = (gemm_alone, gemm_signal_alone, consumer_alone, norm)
+        if args.vendor_gemm:
+            fns += (lambda: torch.matmul(A, B.t(), out=Cplain),)
+        for fn in fns:
             timed(fn, K_, W_)
             MM.zero_()
         torch.cuda.synchronize()
@@ -412,6 +415,9 @@ def main():
     ap.add_argument("--kernels-only", action="store_true",
                     help="run each hot kernel alone on one stream and exit: for counter collection, which "
                          "serialises dispatches and would stall a waiter that spins on another queue")
+    ap.add_argument("--vendor-gemm", action="store_true",
+                    help="with --kernels-only: also launch the vendor library's GEMM (torch.matmul) on the same "
+                         "operands, for a counter run of the yardstick")
     ap.add_argument("--steps-only", action="store_true",
                     help="enqueue warmup + steps overlapped steps and exit: for a kernel-trace timeline of the "
                          "steady state")
