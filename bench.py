@@ -307,6 +307,35 @@ def measure(args, workload, compact=False):
         ACC.zero_()
         torch.cuda.synchronize()
 
+    # Link-rate model (large square only).  The stand-in consumer runs at HBM speed; the collective it stands in for
+    # is bound by the links.  With a rate set on the handle every consumer launch is followed by a kernel that holds
+    # its stream for bytes / rate (algorithm bandwidth: message bytes / time of the collective), in the overlapped
+    # step behind each wave's consumer, in the serial step behind the whole-C consumer: the comparison of
+    # test/test.py:325-371 with the link time modelled instead of measured.  Alternating rounds, medians.
+    link_model = []
+    rates = [float(x) for x in args.link_gbps.split(",") if x] if workload == "c5" and not W and not args.no_group_sweep else []
+    for rate in rates:
+        ns_all = int(2.0 * M * N / rate)
+
+        def serial_link():
+            ops.gemm(A, B, Cplain, algo)
+            ops.consumer_reduce(Cplain.view(-1), ACC)
+            ops.pace(ns_all)
+            ops.rmsnorm(Cplain, Y, gamma, eps=eps)
+
+        ov.set_link_rate(rate)
+        sl = {"overlapped": [], "serial": []}
+        for _ in range(3):
+            sl["overlapped"].append(timed(step_overlapped, K_, W_)[0])
+            sl["serial"].append(timed(serial_link, K_, W_)[0])
+        ov.set_link_rate(0)
+        mo, msr = statistics.median(sl["overlapped"]), statistics.median(sl["serial"])
+        link_model.append({"link_GBps": rate, "link_ms_whole_C": ns_all * 1e-6, "overlapped_ms": mo, "serial_ms": msr,
+                           "overlapped_vs_serial": mo / msr, "speedup": msr / mo})
+    if rates:
+        ACC.zero_()
+        torch.cuda.synchronize()
+
     # bf16 repeat of the large square: the same step with bf16 operands
     bf16_repeat = None
     if workload == "c5" and dt == "f16" and not args.no_group_sweep:
@@ -386,6 +415,9 @@ def measure(args, workload, compact=False):
         "reorder_rmsnorm_GBps": (4.0 * bs * N + 2.0 * N) / (ms_norm * 1e-3) / 1e9,
         "hbm_peak_GBps": PEAK_HBM_GBS,
         "group_sweep": sweep,
+        "link_model": {"what": "the same overlapped and serial step with a modelled link time (bytes / rate) behind "
+                               "every consumer launch; a model of a link-bound collective on one GPU, not a measurement "
+                               "of one", "rates": link_model} if link_model else None,
         "bf16_repeat": bf16_repeat,
     }
 
@@ -410,6 +442,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--group-tiles", type=int, default=0, help="tiles per wave group (0: the workload's default)")
     ap.add_argument("--no-group-sweep", action="store_true", help="skip the wave-group-size sweep (c5 only)")
+    ap.add_argument("--link-gbps", default="100,200,400",
+                    help="link-rate model (c5 only): algorithm bandwidths, in GB/s, of the collective the consumer "
+                         "stands in for; empty: skip")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="skip the compact records of the c2, c3 and c4 workloads that the default c5 run appends")
     ap.add_argument("--kernels-only", action="store_true",

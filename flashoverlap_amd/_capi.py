@@ -53,6 +53,8 @@ SIGNATURES = {
     "fo_overlap_set_accumulator": (c_int, [vp, vp, c_i64]),
     "fo_overlap_set_fused_consumer": (c_int, [vp, c_int]),
     "fo_overlap_set_schedule": (c_int, [vp, ctypes.c_double, c_int]),
+    "fo_overlap_set_link_rate": (c_int, [vp, ctypes.c_double]),
+    "fo_pace": (c_int, [c_i64, vp]),
     "fo_overlap_set_wait_limit": (c_int, [vp, c_i64]),
     "fo_overlap_status": (c_int, [vp, vp]),
     "fo_overlap_comm_stream": (vp, [vp]),

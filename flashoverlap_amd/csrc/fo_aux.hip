@@ -818,6 +818,42 @@ extern "C" int fo_wait_bounded(int expect, int32_t *counter, int64_t max_polls, 
     return fo_wait_with(expect, counter, (long)max_polls, status, stream);
 }
 
+// Holds a stream for a stretch of time: the link time of a collective in the link-rate model of the
+// overlap handle (fo_overlap_set_link_rate).  One lane reads the constant-rate clock and sleeps between
+// reads; it touches no memory and always ends (the clock advances, the host caps the stretch).
+namespace {
+__global__ void fo_pace_kernel(long long ticks) {
+    const long long t0 = wall_clock64();
+    while ((long long)wall_clock64() - t0 < ticks) __builtin_amdgcn_s_sleep(32);
+}
+constexpr double kMaxPaceSeconds = 1.0;
+}  // namespace
+
+int fo_pace_with(double seconds, fo_stream_t stream) {
+    if (!(seconds >= 0)) return FO_ERR_ARG;
+    if (seconds > kMaxPaceSeconds) return FO_ERR_LIMIT;
+    static int khz[64];  // ticks of wall_clock64 per millisecond, per device
+    int dev = 0;
+    FO_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64) return FO_ERR_STATE;
+    if (!khz[dev]) {
+        int rate = 0;
+        FO_HIP_CHECK(hipDeviceGetAttribute(&rate, hipDeviceAttributeWallClockRate, dev));
+        if (rate <= 0) return FO_ERR_STATE;
+        khz[dev] = rate;
+    }
+    const long long ticks = (long long)(seconds * 1e3 * khz[dev]);
+    if (ticks <= 0) return FO_OK;
+    hipLaunchKernelGGL(fo_pace_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream), ticks);
+    FO_LAUNCH_CHECK();
+    return FO_OK;
+}
+
+extern "C" int fo_pace(int64_t nanoseconds, fo_stream_t stream) {
+    if (nanoseconds < 0) return FO_ERR_ARG;
+    return fo_pace_with(nanoseconds * 1e-9, stream);
+}
+
 // Fills n words; the clearing step of callers that may be under stream capture,
 // where a memset node is avoided.
 namespace {

@@ -57,17 +57,24 @@ struct fo_overlap {
     double in_stream_below_flop = kInStreamBelowFlop;
     int token = 1;         // value the fork and join words carry from one stream to the other
     bool always_fork = false;  // the consumer stream must not start before this call's first kernel on the GEMM stream
+    // Link-rate model (fo_overlap_set_link_rate): bytes per second a collective over the group's bytes would
+    // sustain; 0: none.  With a rate every consumer launch is followed on its stream by a kernel that holds the
+    // stream for the bytes' link time, so that the schedule can be timed against a link-bound collective on
+    // one GPU.
+    double link_bytes_per_s = 0;
 };
 
 namespace {
 
+// With a link rate the automatic choices go to per-wave launches on the second stream: the link time
+// follows each consumer launch, and it is what the second stream is there to hide.
 bool in_stream(const fo_overlap *h, int M, int N, int K) {
     if (!h->comm_stream) return true;
-    return h->fused < 0 && 2.0 * M * N * K < h->in_stream_below_flop;
+    return h->fused < 0 && h->link_bytes_per_s <= 0 && 2.0 * M * N * K < h->in_stream_below_flop;
 }
 
 int fused_grid(const fo_overlap *h, int G) {  // 0: per-group launches, otherwise workgroups of the one launch
-    if (h->fused < 0) return G > h->fused_from_groups ? 256 : 0;
+    if (h->fused < 0) return G > h->fused_from_groups && h->link_bytes_per_s <= 0 ? 256 : 0;
     if (h->fused == 1) return 256;
     return h->fused;
 }
@@ -105,6 +112,12 @@ int batch_end(const int32_t *cseg_host, int G, int i, long done, int wave) {
     long d = done + cseg_host[i];
     while (j < G && (d + cseg_host[j] - 1) / wave == w) d += cseg_host[j++];
     return j;
+}
+
+// Link time of `bytes` on `stream` (nothing without a rate).
+int link_time(const fo_overlap *h, int64_t bytes, fo_stream_t stream) {
+    if (h->link_bytes_per_s <= 0 || bytes <= 0) return FO_OK;
+    return fo_pace_with((double)bytes / h->link_bytes_per_s, stream);
 }
 
 int check_segments(const int32_t *cseg_host, int G, long tiles) {
@@ -261,6 +274,12 @@ extern "C" int fo_overlap_set_schedule(fo_overlap_t *h, double in_stream_below_f
     return FO_OK;
 }
 
+extern "C" int fo_overlap_set_link_rate(fo_overlap_t *h, double gigabytes_per_second) {
+    if (!h || !(gigabytes_per_second >= 0)) return FO_ERR_ARG;
+    h->link_bytes_per_s = gigabytes_per_second * 1e9;
+    return FO_OK;
+}
+
 extern "C" int fo_overlap_status(fo_overlap_t *h, int32_t *gave_up) {
     if (!h || !gave_up) return FO_ERR_ARG;
     *gave_up = 0;
@@ -388,6 +407,8 @@ int allreduce_overlap(fo_overlap *h, int dtype, int M, int N, int K, const void 
                                         h->workspace, fused, fused_slices((int64_t)M * N, G, fused),
                                         fused_poll_gap_ns(M, N, K, fused), stream_acc, h->max_polls, h->comm_stream);
         if (rc) return rc;
+        rc = link_time(h, (int64_t)M * N * 2, h->comm_stream);
+        if (rc) return rc;
         if (np) {  // that launch ends when the last group has been consumed: every row at once
             rc = norm_tile_rows(*np, dtype, C, M, N, info[0], info[1], rLDN, RA, 0, TM, false, h->comm_stream);
             if (rc) return rc;
@@ -413,6 +434,8 @@ int allreduce_overlap(fo_overlap *h, int dtype, int M, int N, int K, const void 
                                              j < G && !same_stream);  // every batch but the last runs beside the GEMM
                 if (rc) return rc;
             }
+            rc = link_time(h, n * 2, cstream);
+            if (rc) return rc;
             off += n;
             done += tiles;
             if (np) {
@@ -511,11 +534,14 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
                                         fused_slices((int64_t)M * N, G, fused), fused_poll_gap_ns(M, N, K, fused),
                                         stream_acc, h->max_polls, cstream);
         if (rc) return rc;
+        rc = link_time(h, (int64_t)M * N * 2, cstream);
+        if (rc) return rc;
     }
     int64_t off = 0;
     long done = 0;
     for (int i = 0; i < G;) {
         const int j = fused ? i + 1 : batch_end(cseg_host, G, i, done, wave);
+        const int64_t off_batch = off;
         if (!fused && !quiet) {
             int32_t *gave_up = h->workspace ? h->workspace + kWsGaveUp : nullptr;
             rc = j - i == 1 ? fo_wait_with(cseg_host[i], MM + i, h->max_polls, gave_up, cstream)
@@ -546,6 +572,10 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
             off += n;
             done += cseg_host[g];
         }
+        if (!fused) {
+            rc = link_time(h, (off - off_batch) * 2, cstream);
+            if (rc) return rc;
+        }
         i = j;
     }
     return same_stream ? FO_OK : join(h, captured);
@@ -558,8 +588,11 @@ extern "C" int fo_overlap_gemm_allreduce_serial(fo_overlap_t *h, int dtype, int 
     if (h->acc && h->acc_nelem < (int64_t)M * N) return FO_ERR_ARG;
     int rc = fo_gemm(dtype, M, N, K, A, B, C, algo, h->gemm_stream);
     if (rc) return rc;
-    if (h->acc) return fo_consumer_reduce(dtype, C, h->acc, (int64_t)M * N, h->gemm_stream);
-    return FO_OK;
+    if (h->acc) {
+        rc = fo_consumer_reduce(dtype, C, h->acc, (int64_t)M * N, h->gemm_stream);
+        if (rc) return rc;
+    }
+    return link_time(h, (int64_t)M * N * 2, h->gemm_stream);
 }
 
 extern "C" int fo_overlap_seg_allreduce(fo_overlap_t *h, int dtype, void *C, int64_t MN,
@@ -579,6 +612,8 @@ extern "C" int fo_overlap_seg_allreduce(fo_overlap_t *h, int dtype, void *C, int
             int rc = fo_consumer_reduce(dtype, c + off, acc + off, n, h->gemm_stream);
             if (rc) return rc;
         }
+        int rc = link_time(h, n * 2, h->gemm_stream);
+        if (rc) return rc;
         off += n;
     }
     return FO_OK;

@@ -218,6 +218,10 @@ struct OverlapImpl : torch::CustomClassHolder {
     void set_fused_consumer(int64_t fused) {
         check(fo_overlap_set_fused_consumer(h, (int)fused), "set_fused_consumer");
     }
+    // addition: link-rate model, gigabytes per second of the collective the consumer stands in for (0: off).
+    void set_link_rate(double gigabytes_per_second) {
+        check(fo_overlap_set_link_rate(h, gigabytes_per_second), "set_link_rate");
+    }
     // addition: whether a bounded device-side wait gave up since the last query (synchronises).
     int64_t status() {
         int32_t gave_up = 0;
@@ -260,16 +264,24 @@ struct BaselineImpl : torch::CustomClassHolder {
         gemm_allreduce(A, B, C);
     }
     void nccl_allreduce(at::Tensor C) {
-        if (!acc.defined()) return;
-        TORCH_CHECK(acc.numel() >= C.numel() && acc.scalar_type() == C.scalar_type(),
-                    "flashoverlap: the accumulator must hold C.numel() elements of C's dtype");
-        check(fo_consumer_reduce(dtype_of(C), dev_ptr(C, "C"), acc.data_ptr(), C.numel(),
-                                 current_stream()),
-              "nccl_allreduce");
+        if (acc.defined()) {
+            TORCH_CHECK(acc.numel() >= C.numel() && acc.scalar_type() == C.scalar_type(),
+                        "flashoverlap: the accumulator must hold C.numel() elements of C's dtype");
+            check(fo_consumer_reduce(dtype_of(C), dev_ptr(C, "C"), acc.data_ptr(), C.numel(),
+                                     current_stream()),
+                  "nccl_allreduce");
+        }
+        if (link_gb_per_s > 0)  // the same link time the overlapped calls model (OverlapImpl.set_link_rate)
+            check(fo_pace((int64_t)(C.numel() * C.element_size() / link_gb_per_s), current_stream()), "nccl_allreduce");
     }
     void nccl_reducescatter(at::Tensor /*C*/) {}
     void nccl_all2all(at::Tensor /*C*/, at::Tensor /*D*/, at::Tensor /*mLen_CPU*/) {}
     void set_accumulator(at::Tensor ACC) { acc = ACC; }  // addition
+    double link_gb_per_s = 0;
+    void set_link_rate(double gigabytes_per_second) {  // addition
+        TORCH_CHECK(gigabytes_per_second >= 0, "flashoverlap: the link rate must not be negative");
+        link_gb_per_s = gigabytes_per_second;
+    }
 };
 
 // generate_nccl_id, src/nccl_utils.cu:7-14: 128 opaque bytes as 16 int64.  No
@@ -323,6 +335,7 @@ TORCH_LIBRARY(flashoverlap_class, m) {
         .def("gemm_reducescatter", &BaselineImpl::gemm_reducescatter)
         .def("gemm_all2all", &BaselineImpl::gemm_all2all)
         .def("cublas_gemm", &BaselineImpl::cublas_gemm)
+        .def("set_link_rate", &BaselineImpl::set_link_rate)
         .def("nccl_allreduce", &BaselineImpl::nccl_allreduce)
         .def("nccl_reducescatter", &BaselineImpl::nccl_reducescatter)
         .def("nccl_all2all", &BaselineImpl::nccl_all2all)
@@ -346,6 +359,7 @@ TORCH_LIBRARY(flashoverlap_class, m) {
         .def("set_accumulator", &OverlapImpl::set_accumulator)
         .def("clear_accumulator", &OverlapImpl::clear_accumulator)
         .def("set_fused_consumer", &OverlapImpl::set_fused_consumer)
+        .def("set_link_rate", &OverlapImpl::set_link_rate)
         .def("status", &OverlapImpl::status);
 }
 

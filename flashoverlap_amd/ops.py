@@ -121,6 +121,11 @@ def wait_bounded(expect, MM, index, max_polls, status, stream=None):
                                 _i32(status, "status"), _stream(stream)), "fo_wait_bounded")
 
 
+def pace(nanoseconds, stream=None):
+    """Holds the stream for the given time (the kernel of the link-rate model alone)."""
+    check(lib().fo_pace(int(nanoseconds), _stream(stream)), "fo_pace")
+
+
 def _same_dtype(*tensors):
     if len({t.dtype for t in tensors if t is not None}) > 1:
         raise TypeError("all value tensors of a call must share one dtype")
@@ -257,6 +262,11 @@ class Overlap:
     def set_schedule(self, in_stream_below_flop=-1.0, fused_from_groups=-1):
         check(lib().fo_overlap_set_schedule(self._h, float(in_stream_below_flop), int(fused_from_groups)),
               "fo_overlap_set_schedule")
+
+    def set_link_rate(self, gigabytes_per_second):
+        """Link-rate model: every consumer launch of this handle's calls is followed by a kernel that holds
+        its stream for bytes / rate, the link time of the collective it stands in for (0: off)."""
+        check(lib().fo_overlap_set_link_rate(self._h, float(gigabytes_per_second)), "fo_overlap_set_link_rate")
 
     def set_wait_limit(self, max_polls):
         """Bound of every device-side wait of this handle's calls (-1: FO_WAIT_MAX_POLLS, 0: none)."""

@@ -7,7 +7,10 @@ BaselineImpl.gemm_allreduce / gemm_reducescatter, src/baseline_impl.cu:84-96),
 and prints the reference's table.  Warm-up 20, 200 repetitions, per-call device
 events, mean (test/test.py:17-18, :112-119).
 
-    python -m flashoverlap_amd.speed --m 4096 --n 8192 --k 8192 [--comm_op reduce_scatter --world 8]
+    python -m flashoverlap_amd.speed --m 4096 --n 8192 --k 8192 [--comm_op reduce_scatter --world 8] [--link_gbps 200]
+
+--link_gbps R times all three under the link-rate model (Overlap.set_link_rate): every consumer launch is
+followed by bytes / R of link time, as a collective of that algorithm bandwidth would take.
 """
 import argparse
 
@@ -31,7 +34,8 @@ def _mean_ms(fn, warmup=WARM_UP, reps=REP):
     return float(torch.tensor([s.elapsed_time(e) for s, e in zip(start, end)]).mean())
 
 
-def measure(M, N, K, data, comm_op="all_reduce", world=1, dtype=torch.float16, warmup=WARM_UP, reps=REP):
+def measure(M, N, K, data, comm_op="all_reduce", world=1, dtype=torch.float16, warmup=WARM_UP, reps=REP,
+            link_gbps=0.0):
     """Returns (comm_ms, overlap_ms, baseline_ms) for one stage-2 config dict."""
     BM, BN, algo, cseg, hint = data["BM"], data["BN"], data["Algo"], data["cSeg"], data["hint"]
     TM, TN = M // BM, N // BN
@@ -50,13 +54,17 @@ def measure(M, N, K, data, comm_op="all_reduce", world=1, dtype=torch.float16, w
     cs_gpu = cs_cpu.cuda()
     ov = ops.Overlap(rank=0, world=W)
     ov.set_accumulator(ACC)
+    ov.set_link_rate(link_gbps)
     seg = (M // W) * N
+    link_ns = int(2.0 * M * N / link_gbps) if link_gbps > 0 else 0
 
     def consumer_all(src):
         if rs and W > 1:
             ops.consumer_reduce_rs(src, ACC, W, seg)
         else:
             ops.consumer_reduce(src, ACC)
+        if link_ns:
+            ops.pace(link_ns)
 
     def overlapped():
         if len(cseg) == 1:            # one group: no overlap, as test/test.py:104-133
@@ -87,10 +95,11 @@ def main(argv=None):
     ap.add_argument("--world", type=int, default=8, help="chunks of the emulated reduce-scatter layout")
     ap.add_argument("--dtype", default="f16", choices=["f16", "bf16"])
     ap.add_argument("--path", default=None, help="directory of the config JSONs")
+    ap.add_argument("--link_gbps", type=float, default=0.0, help="link-rate model: algorithm bandwidth of the collective")
     a = ap.parse_args(argv)
     data = config.load_solution(a.m, a.n, a.k, directory=a.path)
     dtype = torch.float16 if a.dtype == "f16" else torch.bfloat16
-    comm, over, base = measure(a.m, a.n, a.k, data, a.comm_op, a.world, dtype)
+    comm, over, base = measure(a.m, a.n, a.k, data, a.comm_op, a.world, dtype, link_gbps=a.link_gbps)
     tile_num = a.m // data["BM"] * a.n // data["BN"]
     rows = [("m", a.m), ("n", a.n), ("k", a.k), ("tile_num", tile_num),
             ("wave_tiles", _capi.wave_tiles(data["Algo"], a.m, a.n)), ("groups", len(data["cSeg"]))]

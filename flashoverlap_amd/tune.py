@@ -138,15 +138,18 @@ def profile_gemm_configs(M, N, K, dtype=torch.float16, top=10, warmup=10, reps=1
     return [r[1] for r in rows], [r[2] for r in rows], [r[0] for r in rows], [r[3] for r in rows]
 
 
-def consumer_bandwidth_curve(dtype=torch.float16, points=36, warmup=5, reps=20):
+def consumer_bandwidth_curve(dtype=torch.float16, points=36, warmup=5, reps=20, link_gbps=0.0):
     """[points, 2] tensor (elements, GiB/ms) of the consumer over 2^(20+0.25 i)
-    elements -- the one-GPU analogue of tune/bandwidth.py:77-111."""
+    elements -- the one-GPU analogue of tune/bandwidth.py:77-111.  link_gbps > 0: the curve of the
+    link-rate model (Overlap.set_link_rate), i.e. the consumer's time plus 2 n bytes / rate."""
     sizes = [int(2 ** (20 + 0.25 * i)) // 8 * 8 for i in range(points)]
     buf = torch.zeros(max(sizes), device="cuda", dtype=dtype)
     acc = torch.zeros(max(sizes), device="cuda", dtype=dtype)
     out = torch.empty(points, 2, dtype=torch.float64)
     for i, n in enumerate(sizes):
         ms = _time_ms(lambda: ops.consumer_reduce(buf[:n], acc[:n]), warmup, reps)
+        if link_gbps > 0:
+            ms += 2.0 * n / (link_gbps * 1e9) * 1e3
         out[i, 0] = n
         out[i, 1] = n * CONSUMER_BYTES_PER_ELEM / (1024 ** 3) / ms
     return out
@@ -193,7 +196,7 @@ def measured_hint(M, N, K, algo, wave, dtype=torch.float16, warmup=20, samples=1
 
 
 def time_overlap(M, N, K, algo, cseg, hint, dtype=torch.float16, warmup=20, reps=200, fused=False,
-                 with_consumer=True, settle_s=0.2):
+                 with_consumer=True, settle_s=0.2, link_gbps=0.0):
     """Mean ms of the overlapped call for one cSeg (tune/search.py:255-347)."""
     BM, BN = _capi.algo_tile(algo)
     TM, TN = M // BM, N // BN
@@ -206,6 +209,7 @@ def time_overlap(M, N, K, algo, cseg, hint, dtype=torch.float16, warmup=20, reps
     cseg_gpu = cseg_cpu.cuda()
     ov = ops.Overlap()
     ov.set_fused_consumer(fused)
+    ov.set_link_rate(link_gbps)
     if with_consumer:
         ov.set_accumulator(torch.zeros(M * N, device="cuda", dtype=dtype))
     if len(cseg) == 1:
@@ -219,7 +223,7 @@ def time_overlap(M, N, K, algo, cseg, hint, dtype=torch.float16, warmup=20, reps
 
 
 def compare_overlap(M, N, K, algo, csegs, hint, dtype=torch.float16, rounds=2, reps=30, warmup=3,
-                    with_consumer=True):
+                    with_consumer=True, link_gbps=0.0):
     """Median ms of the overlapped call for each cSeg of `csegs`, measured on one set of buffers with
     the candidates taking turns (`rounds` passes over all of them, `reps` timed calls each): what is
     left of clock drift and of one-off disturbances falls on all candidates alike.  For deciding
@@ -232,6 +236,7 @@ def compare_overlap(M, N, K, algo, csegs, hint, dtype=torch.float16, rounds=2, r
     RA = reorder_indices(TM * TN, hint).reshape(TM, TN)
     MM = torch.zeros(counter_size(max(len(c) for c in csegs), TM, TN), dtype=torch.int32, device="cuda")
     ov = ops.Overlap()
+    ov.set_link_rate(link_gbps)
     if with_consumer:
         ov.set_accumulator(torch.zeros(M * N, device="cuda", dtype=dtype))
     calls = []
@@ -263,14 +268,14 @@ def compare_overlap(M, N, K, algo, csegs, hint, dtype=torch.float16, rounds=2, r
     return [float(np.median(x)) for x in samples]
 
 
-def exhaustive_search(M, N, K, algo, wave, hint, dtype=torch.float16, reps=50):
+def exhaustive_search(M, N, K, algo, wave, hint, dtype=torch.float16, reps=50, link_gbps=0.0):
     """Measure every composition of the wave count (tune/search.py:387-439)."""
     BM, BN = _capi.algo_tile(algo)
     tile_num = (M // BM) * (N // BN)
     best, best_ms, table = None, float("inf"), []
     for gp in integer_partitions(div_up(tile_num, wave)):
         cseg = groups_to_cseg(gp, wave, tile_num)
-        ms = time_overlap(M, N, K, algo, cseg, hint, dtype, warmup=5, reps=reps)
+        ms = time_overlap(M, N, K, algo, cseg, hint, dtype, warmup=5, reps=reps, link_gbps=link_gbps)
         table.append((cseg, ms))
         if ms < best_ms:
             best, best_ms = cseg, ms
@@ -306,10 +311,12 @@ def choose_candidate(M, N, K, BMs, BNs, algos, predictive, dtype=torch.float16, 
 
 # ------------------------------------------------------------------ command line
 def tune_shape(M, N, K, comm_op="all_reduce", predictive=False, dtype=torch.float16, directory=None,
-               candidates=None, reps=100, quiet=False):
+               candidates=None, reps=100, quiet=False, link_gbps=0.0):
     """The reference's three tuning steps for one shape on one GPU, writing the same
     JSON files: GEMM candidates (tune/gen_config.py), consumer bandwidth curve
-    (tune/bandwidth.py), wave-group search (tune/search.py).  Returns the solution dict."""
+    (tune/bandwidth.py), wave-group search (tune/search.py).  Returns the solution dict.
+    link_gbps > 0 tunes for the link-rate model (a collective of that algorithm bandwidth) instead of
+    the consumer alone."""
     import os
     from . import config
     say = (lambda *a: None) if quiet else print
@@ -320,7 +327,7 @@ def tune_shape(M, N, K, comm_op="all_reduce", predictive=False, dtype=torch.floa
     predictive = predictive or M * N > 33554432
     curve = None
     if predictive:
-        curve = consumer_bandwidth_curve(dtype)
+        curve = consumer_bandwidth_curve(dtype, link_gbps=link_gbps)
         cdir = directory or config.DEFAULT_DIR
         os.makedirs(cdir, exist_ok=True)
         torch.save(curve, os.path.join(cdir, f"bandwidth_{comm_op}_tp1.pt"))
@@ -334,10 +341,11 @@ def tune_shape(M, N, K, comm_op="all_reduce", predictive=False, dtype=torch.floa
         cseg, est = predictive_search(M, N, dur, curve.numpy(), tile_num, wave)
         say("predicted latency %.4f ms for cSeg %s" % (est, cseg))
     else:
-        cseg, ms, table = exhaustive_search(M, N, K, algo, wave, hint, dtype, reps=max(10, reps // 4))
+        cseg, ms, table = exhaustive_search(M, N, K, algo, wave, hint, dtype, reps=max(10, reps // 4),
+                                            link_gbps=link_gbps)
         for c, c_ms in table:
             say(c, "%.4f" % c_ms)
-    ms = time_overlap(M, N, K, algo, cseg, hint, dtype, warmup=10, reps=reps)
+    ms = time_overlap(M, N, K, algo, cseg, hint, dtype, warmup=10, reps=reps, link_gbps=link_gbps)
     say("searched latency %.4f ms, best cSeg %s" % (ms, cseg))
     path = config.save_solution(M, N, K, BM, BN, dur, algo, hint, cseg, directory=directory)
     say("solution ->", path)
@@ -354,9 +362,11 @@ def main(argv=None):
     ap.add_argument("--predictive_search", type=bool, default=False)  # any non-empty string is true, as in the reference
     ap.add_argument("--dtype", default="f16", choices=["f16", "bf16"])
     ap.add_argument("--path", default=None, help="directory of the config JSONs")
+    ap.add_argument("--link_gbps", type=float, default=0.0,
+                    help="tune for a collective of this algorithm bandwidth (link-rate model) instead of the consumer alone")
     a = ap.parse_args(argv)
     tune_shape(a.m, a.n, a.k, a.comm_op, a.predictive_search,
-               torch.float16 if a.dtype == "f16" else torch.bfloat16, a.path)
+               torch.float16 if a.dtype == "f16" else torch.bfloat16, a.path, link_gbps=a.link_gbps)
 
 
 if __name__ == "__main__":

@@ -294,6 +294,23 @@ int fo_overlap_set_fused_consumer(fo_overlap_t *h, int fused);
  * than fused_from_groups groups get the one-launch consumer.  The defaults
  * (6.4e10, 16) were measured on one MI355X; a negative value restores one. */
 int fo_overlap_set_schedule(fo_overlap_t *h, double in_stream_below_flop, int fused_from_groups);
+/* Link-rate model (no counterpart in the reference, where the collective is
+ * NCCL's and takes what the links give it: src/overlap_impl.cu:256, :312-313;
+ * the tuner measures that rate into its bandwidth curve, tune/bandwidth.py:77-111).
+ * On one GPU the consumer that stands in for the collective runs at HBM speed,
+ * twenty to fifty times faster than a collective over the links, and there is
+ * little for the schedule to hide.  With gigabytes_per_second > 0 every consumer
+ * launch of the handle's calls (overlapped and serial ones alike) is followed, on
+ * the same stream, by a one-lane kernel that holds the stream for
+ * bytes of C in the launch / rate: the time the collective would spend on the links
+ * at that algorithm bandwidth.  Results do not change.  The automatic choices then
+ * go to per-wave launches on the second stream.  0 (default) switches it off.
+ * A single stretch above one second returns FO_ERR_LIMIT from the call. */
+int fo_overlap_set_link_rate(fo_overlap_t *h, double gigabytes_per_second);
+/* The kernel of that model alone: holds `stream` for the given time (at most one
+ * second; it reads the device's constant-rate clock, touches no memory and
+ * always ends). */
+int fo_pace(int64_t nanoseconds, fo_stream_t stream);
 /* Bound, in polls, of every device-side wait the handle's calls enqueue
  * (group waits, the one-launch consumer's polls, fork and join): -1 (default)
  * takes FO_WAIT_MAX_POLLS from the environment, 0 waits without bound like

@@ -482,6 +482,35 @@ def test_predictive_search_on_measured_curve(fo):
     assert sum(cseg) == 2048 and est > 0.4
 
 
+def test_predictive_search_under_the_link_rate_model(fo):
+    """With a link-bound collective behind the consumer (Overlap.set_link_rate, 200 GB/s: the whole C takes
+    0.67 ms, three times the GEMM) the splits differ by tens of percent, and the predictive search
+    (tune/search.py:442-502) on the curve of that model must pick one that measures within 5 % of the best
+    of all eight compositions of the four waves, clearly below the single group, and near its own estimate."""
+    from flashoverlap_amd import tune
+    link = 200.0
+    curve = tune.consumer_bandwidth_curve(points=36, warmup=2, reps=5, link_gbps=link).numpy()
+    M, N, K = 8192, 8192, 2048
+    algo = fo._capi.find_algo(256, 128, swizzle=4)
+    T, wave = 2048, fo._capi.wave_tiles(algo, M, N)
+    assert wave == 512
+    A = torch.randn(M, K, device="cuda").half()
+    B = torch.randn(N, K, device="cuda").half()
+    C = torch.empty(M, N, device="cuda", dtype=torch.float16)
+    gemm_ms = tune._time_ms(lambda: fo.ops.gemm(A, B, C, algo), 10, 30, settle_s=0.3)
+    pred, est = tune.predictive_search(M, N, gemm_ms, curve, T, wave)
+    csegs = [tune.groups_to_cseg(gp, wave, T) for gp in tune.integer_partitions(4)]
+    assert pred in csegs and [T] in csegs
+    hint = fo._capi.schedule_order(algo, M, N)
+    times = tune.compare_overlap(M, N, K, algo, csegs, hint, rounds=2, reps=10, warmup=2, link_gbps=link)
+    t_pred, t_single = times[csegs.index(pred)], times[csegs.index([T])]
+    report = {tuple(c): round(t, 4) for c, t in zip(csegs, times)}
+    assert t_single >= 2.0 * M * N / (link * 1e9) * 1e3 + gemm_ms * 0.9, report   # nothing hidden: GEMM + link time
+    assert t_pred <= min(times) * 1.05, (pred, report)
+    assert t_pred <= t_single * 0.9, (pred, report)
+    assert abs(est - t_pred) <= 0.15 * t_pred, (pred, est, report)
+
+
 def test_predictive_search_against_checker_and_measurement(fo, oracle):
     """The latency model evaluated on the *measured* consumer curve must be the checker's
     (tune/search.py:207-235), the predictive choice must be the checker's argmin over the same

@@ -212,3 +212,58 @@ def test_dropin_class_exposes_the_call(fo):
     fo.ops.reorder_rmsnorm_rows(plain, Y_plain, gamma, 0, M, 1, 8, 1, None, eps=EPS)
     torch.cuda.synchronize()
     assert torch.equal(Y, Y_plain) and (MM == 0).all() and impl.status() == 0
+
+
+def test_link_rate_model_holds_the_consumer_stream_and_changes_no_result(fo):
+    """fo_overlap_set_link_rate: every consumer launch is followed by a kernel that holds its stream for
+    bytes / rate.  Results are those of the call without it; the call takes at least the link time of the
+    last wave's bytes longer than the GEMM, and the serial call at least the whole matrix's link time."""
+    dtype, bm, bn, M, N, K = F16, 128, 256, 2048, 4096, 1024
+    T = (M // bm) * (N // bn)
+    cseg = [T // 4] * 4
+    algo, RA, A, B, gamma, MM, cs_cpu, cs_gpu = _setup(fo, dtype, bm, bn, M, N, K, cseg, 31)
+    td = TORCH_DTYPE[dtype]
+    acc0, _ = seeded((M * N,), dtype, 34, scale=0.5)
+    RA_cpu = RA.cpu()
+    ov = fo.ops.Overlap()
+    ov.set_fused_consumer(0)
+    out = {}
+    for rate in (0.0, 20.0):          # 16.8 MB of C at 20 GB/s: 0.84 ms of link time
+        C = torch.full((M * N,), float("nan"), device="cuda", dtype=td)
+        Y = torch.full((M, N), float("nan"), device="cuda", dtype=td)
+        acc = acc0.clone()
+        ov.set_accumulator(acc)
+        ov.set_link_rate(rate)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ov.gemm_allreduce_rmsnorm_overlap(A, B, C, MM, RA, RA_cpu, 1, cs_cpu, cs_gpu, algo, Y, gamma, eps=EPS)
+        torch.cuda.synchronize()
+        e0.record()
+        ov.gemm_allreduce_rmsnorm_overlap(A, B, C, MM, RA, RA_cpu, 1, cs_cpu, cs_gpu, algo, Y, gamma, eps=EPS)
+        e1.record()
+        torch.cuda.synchronize()
+        assert ov.status() == 0 and (MM == 0).all()
+        out[rate] = (C, Y, acc, e0.elapsed_time(e1))
+    assert torch.equal(out[0.0][0], out[20.0][0]) and torch.equal(out[0.0][1], out[20.0][1])
+    assert torch.equal(out[0.0][2], out[20.0][2])
+    link_ms = 2.0 * M * N / 20e9 * 1e3
+    assert out[20.0][3] >= link_ms * 0.95 and out[0.0][3] < link_ms * 0.5, (out[0.0][3], out[20.0][3], link_ms)
+    # the serial comparator of the handle models the same link
+    Cs = torch.empty(M, N, device="cuda", dtype=td)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    ov.gemm_allreduce(A, B, Cs, algo)
+    e1.record()
+    torch.cuda.synchronize()
+    assert e0.elapsed_time(e1) >= link_ms * 0.95
+    # the kernel alone, and its limit
+    e0.record()
+    fo.ops.pace(300_000)
+    e1.record()
+    torch.cuda.synchronize()
+    assert 0.28 <= e0.elapsed_time(e1) < 1.0
+    with pytest.raises(RuntimeError):
+        fo.ops.pace(2_000_000_000)
+    with pytest.raises(RuntimeError):
+        ov.set_link_rate(-1.0)
+    ov.set_link_rate(0)
+    ov.close()
