@@ -442,7 +442,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--group-tiles", type=int, default=0, help="tiles per wave group (0: the workload's default)")
     ap.add_argument("--no-group-sweep", action="store_true", help="skip the wave-group-size sweep (c5 only)")
-    ap.add_argument("--link-gbps", default="100,200,400",
+    ap.add_argument("--link-gbps", default="100,200,400,1000",
                     help="link-rate model (c5 only): algorithm bandwidths, in GB/s, of the collective the consumer "
                          "stands in for; empty: skip")
     ap.add_argument("--no-other-workloads", action="store_true",
