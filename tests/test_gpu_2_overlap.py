@@ -714,11 +714,13 @@ def test_overlap_on_three_slot_shapes(fo, fused, bm, bn, M, N, K, cseg):
     ov.close()
 
 
-@pytest.mark.parametrize("fused", [0, 1])
-def test_overlapped_step_captured_in_a_hip_graph(fo, fused):
+@pytest.mark.parametrize("fused,one_call", [(0, False), (1, False), (0, True), (1, True)])
+def test_overlapped_step_captured_in_a_hip_graph(fo, fused, one_call):
     """Capture {overlapped GEMM + consumer, reorder+RMSNorm} once, replay it several times with eager
     work and synchronisations in between and new operand values each time; every replay must give
-    what the eager path gives.  Under capture the two streams are tied by events (graph edges)."""
+    what the eager path gives.  Under capture the two streams are tied by events (graph edges).
+    one_call: the call that enqueues the normalisation itself, on the consumer stream, here also with the
+    link-rate model's kernel behind each consumer launch."""
     M, N, K, bm, bn = 2048, 2048, 256, 128, 128
     cseg = [64] * 4
     algo, RA, A, B, _, _, MM, cs_cpu, cs_gpu = _setup(fo, F16, bm, bn, M, N, K, cseg, swizzle=4, seed=120)
@@ -733,10 +735,16 @@ def test_overlapped_step_captured_in_a_hip_graph(fo, fused):
         ov = ops.Overlap()                    # GEMM stream = s
         ov.set_accumulator(ACC)
         ov.set_fused_consumer(fused)
+        RA_cpu = RA.cpu()
+        if one_call:
+            ov.set_link_rate(400.0)           # 8 MB of C: 21 us per replay
 
         def step():
-            ov.gemm_allreduce_overlap(A, B, Cp, MM, RA, 1, cs_cpu, cs_gpu, algo)
-            ops.reorder_rmsnorm(Cp.view(M, N), Y, gamma, bm, bn, 1, RA, eps=1e-6)
+            if one_call:
+                ov.gemm_allreduce_rmsnorm_overlap(A, B, Cp, MM, RA, RA_cpu, 1, cs_cpu, cs_gpu, algo, Y, gamma, eps=1e-6)
+            else:
+                ov.gemm_allreduce_overlap(A, B, Cp, MM, RA, 1, cs_cpu, cs_gpu, algo)
+                ops.reorder_rmsnorm(Cp.view(M, N), Y, gamma, bm, bn, 1, RA, eps=1e-6)
 
         step()                                # eager warm-up: one-time kernel attribute set-up
     torch.cuda.synchronize()
@@ -756,7 +764,10 @@ def test_overlapped_step_captured_in_a_hip_graph(fo, fused):
         graph.replay()
         torch.cuda.synchronize()
         ops.gemm(A, B, plain, algo)
-        ops.rmsnorm(plain, y_ref, gamma, eps=1e-6)
+        if one_call:  # the row kernel sums a row's squares in another order than the wavefront-per-row kernel
+            ops.reorder_rmsnorm_rows(plain, y_ref, gamma, 0, M, 1, 8, 1, None, eps=1e-6)
+        else:
+            ops.rmsnorm(plain, y_ref, gamma, eps=1e-6)
         torch.cuda.synchronize()
         assert torch.equal(fo.layout.unpermute(Cp, M, N, bm, bn, RA), plain), f"replay {it}"
         assert torch.equal(Y, y_ref), f"replay {it}"
