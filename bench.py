@@ -31,6 +31,63 @@ MEASURED_TRAFFIC_BYTES = {("c5", "f16"): 788738.0 * 1024 * 2.0 + 131104.0 * 1024
 # against the 2.4 GHz the nominal peak assumes.
 MEASURED_GEMM_COUNTERS = {("c5", "f16"): {"cycles_per_launch": 1.3496e6, "mfma_util": 0.777}}
 
+
+class PowerSampler:
+    """Socket power of the GPU from the amdgpu hwmon files (power1_average or power1_input, microwatts;
+    power1_cap is the limit), read every 10 ms by a thread while a leg loops.  None where the files are
+    missing or unreadable."""
+
+    def __init__(self):
+        import glob
+        self.path = self.cap_w = None
+        for h in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*")):
+            for name in ("power1_average", "power1_input"):
+                f = os.path.join(h, name)
+                try:
+                    int(open(f).read())
+                except (OSError, ValueError):
+                    continue
+                self.path = f
+                try:
+                    self.cap_w = int(open(os.path.join(h, "power1_cap")).read()) / 1e6
+                except (OSError, ValueError):
+                    pass
+                return
+
+    def watts_while(self, fn, seconds, launches_per_sync=50, skip_seconds=0.5):
+        """Mean power while fn loops for `seconds` (the first skip_seconds are left out), and ms per launch."""
+        import threading
+        import torch
+        samples, stop = [], threading.Event()
+
+        def sampler():
+            while not stop.is_set():
+                try:
+                    samples.append((time.perf_counter(), int(open(self.path).read())))
+                except (OSError, ValueError):
+                    pass
+                time.sleep(0.01)
+        th = threading.Thread(target=sampler, daemon=True)
+        t0 = time.perf_counter()
+        if self.path:
+            th.start()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        n = 0
+        e0.record()
+        while time.perf_counter() < t0 + seconds:
+            for _ in range(launches_per_sync):
+                fn()
+            n += launches_per_sync
+            torch.cuda.synchronize()
+        e1.record()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        stop.set()
+        if self.path:
+            th.join()
+        w = [v for (t, v) in samples if t0 + skip_seconds <= t <= t1]
+        return (sum(w) / len(w) / 1e6 if w else None), e0.elapsed_time(e1) / n
+
 WORKLOADS = {
     # name: (M, N, K, BM, BN, dtype, group tiles, W, description)
     "c5": (8192, 8192, 8192, 128, 256, "f16", 256, 0, "large square fp16 8192^3, 128x256 tiles, wave groups of 256 tiles"),
@@ -336,6 +393,32 @@ def measure(args, workload, compact=False):
         ACC.zero_()
         torch.cuda.synchronize()
 
+    # Power (large square only): the GEMM runs at the board's power limit, which is what holds its clock
+    # below the 2.4 GHz of the nominal peak, and an overlapped step cannot finish before the energy of all its
+    # kernels has been delivered at that limit.  Each leg loops for 1.5 s while a thread reads the socket power.
+    power = None
+    if workload == "c5" and not args.no_group_sweep and not W:
+        ps = PowerSampler()
+        if ps.path:
+            pw = {}
+            for name, fn, per_sync in (("gemm_signal", gemm_signal_alone, 50), ("consumer", consumer_alone, 400),
+                                       ("reorder_rmsnorm", norm, 400), ("overlapped_step", step_overlapped, 50),
+                                       ("serial_step", step_serial, 50)):
+                watts, ms = ps.watts_while(fn, 1.5, per_sync)
+                MM.zero_()
+                pw[name] = {"watts": watts, "ms": ms}
+            time.sleep(0.3)
+            idle_w, _ = ps.watts_while(lambda: None, 0.6, 1, skip_seconds=0.2)
+            power = {"source": ps.path, "cap_w": ps.cap_w, "idle_w": idle_w, "legs": pw}
+            if all(v["watts"] for v in pw.values()) and ps.cap_w:
+                # energy above idle of the three kernels run one after the other, delivered at the limit
+                dyn = sum((pw[k]["watts"] - idle_w) * pw[k]["ms"] for k in ("gemm_signal", "consumer", "reorder_rmsnorm"))
+                power["overlapped_step_bound_ms"] = dyn / (ps.cap_w - idle_w)
+                power["bound"] = ("(sum over GEMM, consumer, reorder+RMSNorm of (watts - idle) x ms) / (cap - idle): no "
+                                  "schedule of these three kernels finishes sooner at this power limit")
+            ACC.zero_()
+            torch.cuda.synchronize()
+
     # bf16 repeat of the large square: the same step with bf16 operands
     bf16_repeat = None
     if workload == "c5" and dt == "f16" and not args.no_group_sweep:
@@ -418,8 +501,12 @@ def measure(args, workload, compact=False):
         "link_model": {"what": "the same overlapped and serial step with a modelled link time (bytes / rate) behind "
                                "every consumer launch; a model of a link-bound collective on one GPU, not a measurement "
                                "of one", "rates": link_model} if link_model else None,
+        "power": power,
         "bf16_repeat": bf16_repeat,
     }
+    if power and power["legs"]["gemm_signal"]["watts"]:
+        out["roofline"]["power_w"] = power["legs"]["gemm_signal"]["watts"]
+        out["roofline"]["power_cap_w"] = power["cap_w"]
 
     out["waits_gave_up"] = ov.status()   # 1: a bounded device-side wait ran out of polls; the timings are then void
     return out, ov, (A16, B16, gamma16, eps, M)
