@@ -39,7 +39,7 @@ class PowerSampler:
 
     def __init__(self):
         import glob
-        self.path = self.cap_w = None
+        self.path = self.cap_w = self.sclk_path = self.last_sclk_mhz = None
         for h in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*")):
             for name in ("power1_average", "power1_input"):
                 f = os.path.join(h, name)
@@ -52,20 +52,35 @@ class PowerSampler:
                     self.cap_w = int(open(os.path.join(h, "power1_cap")).read()) / 1e6
                 except (OSError, ValueError):
                     pass
+                self.sclk_path = os.path.join(os.path.dirname(os.path.dirname(h)), "pp_dpm_sclk")
                 return
+
+    def sclk_mhz(self):
+        """The shader clock level the driver marks as current ('1: 1782Mhz *'), or None."""
+        try:
+            for line in open(self.sclk_path):
+                if "*" in line:
+                    return float(line.split(":")[1].lower().split("mhz")[0])
+        except (OSError, ValueError, IndexError, AttributeError):
+            pass
+        return None
 
     def watts_while(self, fn, seconds, launches_per_sync=50, skip_seconds=0.5):
         """Mean power while fn loops for `seconds` (the first skip_seconds are left out), and ms per launch."""
         import threading
         import torch
-        samples, stop = [], threading.Event()
+        samples, clocks, stop = [], [], threading.Event()
 
         def sampler():
+            k = 0
             while not stop.is_set():
                 try:
                     samples.append((time.perf_counter(), int(open(self.path).read())))
                 except (OSError, ValueError):
                     pass
+                if k % 10 == 5:
+                    clocks.append((time.perf_counter(), self.sclk_mhz()))
+                k += 1
                 time.sleep(0.01)
         th = threading.Thread(target=sampler, daemon=True)
         t0 = time.perf_counter()
@@ -86,6 +101,8 @@ class PowerSampler:
         if self.path:
             th.join()
         w = [v for (t, v) in samples if t0 + skip_seconds <= t <= t1]
+        c = [v for (t, v) in clocks if t0 + skip_seconds <= t <= t1 and v]
+        self.last_sclk_mhz = sum(c) / len(c) if c else None
         return (sum(w) / len(w) / 1e6 if w else None), e0.elapsed_time(e1) / n
 
 WORKLOADS = {
@@ -406,7 +423,7 @@ def measure(args, workload, compact=False):
                                        ("serial_step", step_serial, 50)):
                 watts, ms = ps.watts_while(fn, 1.5, per_sync)
                 MM.zero_()
-                pw[name] = {"watts": watts, "ms": ms}
+                pw[name] = {"watts": watts, "ms": ms, "sclk_mhz": ps.last_sclk_mhz}
             time.sleep(0.3)
             idle_w, _ = ps.watts_while(lambda: None, 0.6, 1, skip_seconds=0.2)
             power = {"source": ps.path, "cap_w": ps.cap_w, "idle_w": idle_w, "legs": pw}
