@@ -45,6 +45,7 @@ SIGNATURES = {
     "fo_norm_rows_kernel_info": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, vp]),
     "fo_rmsnorm": (c_int, [c_int, vp, vp, vp, c_int, c_int, c_f32, vp]),
     "fo_overlap_plan_batches": (c_int, [vp, c_int, c_int, vp]),
+    "fo_overlap_plan_norm_rows": (c_int, [vp, c_int, c_int, vp, c_int, c_int, vp, c_int]),
     "fo_overlap_create": (c_int, [ctypes.POINTER(vp)]),
     "fo_overlap_destroy": (c_int, [vp]),
     "fo_overlap_set_gemm_stream": (c_int, [vp, vp]),
@@ -175,6 +176,21 @@ def norm_rows_kernel_info(dim, reorder=True, BN=128, rldn=1, beside_gemm=True, d
     check(lib().fo_norm_rows_kernel_info(int(dtype), int(dim), int(bool(reorder)), int(BN), int(rldn),
                                          int(bool(beside_gemm)), info), "fo_norm_rows_kernel_info")
     return {"vgprs": info[0], "lds_bytes": info[1]}
+
+
+def plan_norm_rows(RA, cseg, wave_tiles):
+    """Schedule of the normalisation inside gemm_allreduce_rmsnorm_overlap: list of (batch, first_tile_row,
+    end_tile_row).  RA: the reorder table as a [TM, TN] array-like on the host."""
+    import numpy as np
+    ra = np.ascontiguousarray(np.asarray(RA, dtype=np.int32))
+    TM, TN = ra.shape
+    G = len(cseg)
+    arr = (ctypes.c_int32 * G)(*cseg)
+    runs = (ctypes.c_int32 * (3 * TM))()
+    n = lib().fo_overlap_plan_norm_rows(ra.ctypes.data_as(ctypes.c_void_p), TM, TN, arr, G, int(wave_tiles), runs, TM)
+    if n < 0:
+        raise FlashOverlapError("fo_overlap_plan_norm_rows", n)
+    return [(runs[3 * i], runs[3 * i + 1], runs[3 * i + 2]) for i in range(n)]
 
 
 def plan_batches(cseg, wave_tiles):

@@ -324,12 +324,12 @@ int norm_tile_rows(const norm_plan &np, int dtype, const void *C, int M, int N, 
 }
 
 // Tile rows whose tiles all lie in storage slots below `done` and that have not been normalised yet, as
-// runs of consecutive tile rows; at most kMaxRuns launches per batch (a reorder table that scatters the rows
-// of a wave leaves the rest to the last batch).  last_slot[tm] = largest slot of tile row tm; -1 once normalised.
+// runs of consecutive tile rows [first, end); at most kMaxRuns runs per batch (a reorder table that scatters the
+// rows of a wave leaves the rest to the last batch, which takes everything that is left).
+// last_slot[tm] = largest slot of tile row tm; -1 once handed out.  Appends to `runs`.
 constexpr int kMaxRuns = 4;
-int norm_ready_rows(const norm_plan &np, long *last_slot, int TM, long done, bool final_batch, int dtype, const void *C,
-                    int M, int N, int BM, int BN, int rLDN, const int32_t *RA, bool beside_gemm, fo_stream_t stream) {
-    int runs = 0;
+void ready_tile_rows(long *last_slot, int TM, long done, bool final_batch, std::vector<int> &runs) {
+    int n = 0;
     for (int tm = 0; tm < TM;) {
         if (last_slot[tm] < 0 || last_slot[tm] >= done) {
             tm++;
@@ -337,12 +337,34 @@ int norm_ready_rows(const norm_plan &np, long *last_slot, int TM, long done, boo
         }
         int end = tm;
         while (end < TM && last_slot[end] >= 0 && last_slot[end] < done) end++;
-        if (!final_batch && runs == kMaxRuns) break;
-        int rc = norm_tile_rows(np, dtype, C, M, N, BM, BN, rLDN, RA, tm, end, beside_gemm, stream);
-        if (rc) return rc;
+        if (!final_batch && n == kMaxRuns) break;
+        runs.push_back(tm);
+        runs.push_back(end);
         for (int t = tm; t < end; t++) last_slot[t] = -1;
-        runs++;
+        n++;
         tm = end;
+    }
+}
+
+// Largest storage slot of every tile row of the reorder table; FO_ERR_ARG for an entry outside [0, TM*TN).
+int last_slots(const int32_t *RA_host, int TM, int TN, std::vector<long> &last_slot) {
+    last_slot.assign(TM, 0);
+    for (int tm = 0; tm < TM; tm++)
+        for (int tn = 0; tn < TN; tn++) {
+            const long r = RA_host[(long)tm * TN + tn];
+            if (r < 0 || r >= (long)TM * TN) return FO_ERR_ARG;
+            if (r > last_slot[tm]) last_slot[tm] = r;
+        }
+    return FO_OK;
+}
+
+int norm_ready_rows(const norm_plan &np, long *last_slot, int TM, long done, bool final_batch, int dtype, const void *C,
+                    int M, int N, int BM, int BN, int rLDN, const int32_t *RA, bool beside_gemm, fo_stream_t stream) {
+    std::vector<int> runs;
+    ready_tile_rows(last_slot, TM, done, final_batch, runs);
+    for (size_t k = 0; k + 1 < runs.size(); k += 2) {
+        int rc = norm_tile_rows(np, dtype, C, M, N, BM, BN, rLDN, RA, runs[k], runs[k + 1], beside_gemm, stream);
+        if (rc) return rc;
     }
     return FO_OK;
 }
@@ -366,13 +388,8 @@ int allreduce_overlap(fo_overlap *h, int dtype, int M, int N, int K, const void 
     if (np) {
         if (!np->Y || !np->Wt || !np->RA_host) return FO_ERR_ARG;
         if (N % 8 || N > 16384 || (int64_t)M * N * 2 > 0xFFFFFFFFLL) return FO_ERR_SHAPE;
-        last_slot.assign(TM, 0);
-        for (int tm = 0; tm < TM; tm++)
-            for (int tn = 0; tn < TN; tn++) {
-                const long r = np->RA_host[(long)tm * TN + tn];
-                if (r < 0 || r >= (long)TM * TN) return FO_ERR_ARG;
-                if (r > last_slot[tm]) last_slot[tm] = r;
-            }
+        rc = last_slots(np->RA_host, TM, TN, last_slot);
+        if (rc) return rc;
     }
 
     const bool same_stream = in_stream(h, M, N, K);
@@ -450,6 +467,35 @@ int allreduce_overlap(fo_overlap *h, int dtype, int M, int N, int K, const void 
 }
 
 }  // namespace
+
+// Which tile rows fo_overlap_gemm_allreduce_norm normalises behind which batch of groups, for a caller that wants
+// to know (and for tests on a machine without a GPU): the same planner the call uses.
+extern "C" int fo_overlap_plan_norm_rows(const int32_t *RA_host, int TM, int TN, const int32_t *cseg_host, int G,
+                                         int wave_tiles, int32_t *runs, int max_runs) {
+    if (!RA_host || !runs || TM <= 0 || TN <= 0 || max_runs <= 0) return FO_ERR_ARG;
+    int rc = check_segments(cseg_host, G, (long)TM * TN);
+    if (rc) return rc;
+    std::vector<long> last_slot;
+    rc = last_slots(RA_host, TM, TN, last_slot);
+    if (rc) return rc;
+    int n = 0, batch = 0;
+    long done = 0;
+    for (int i = 0; i < G; batch++) {
+        const int j = batch_end(cseg_host, G, i, done, wave_tiles);
+        for (int g = i; g < j; g++) done += cseg_host[g];
+        std::vector<int> ready;
+        ready_tile_rows(last_slot.data(), TM, done, j == G, ready);
+        for (size_t k = 0; k + 1 < ready.size(); k += 2) {
+            if (n == max_runs) return FO_ERR_LIMIT;
+            runs[3 * n] = batch;
+            runs[3 * n + 1] = ready[k];
+            runs[3 * n + 2] = ready[k + 1];
+            n++;
+        }
+        i = j;
+    }
+    return n;
+}
 
 extern "C" int fo_overlap_gemm_allreduce(fo_overlap_t *h, int dtype, int M, int N, int K,
                                          const void *A, const void *B, void *C, int32_t *MM,

@@ -278,6 +278,16 @@ int fo_overlap_set_accumulator(fo_overlap_t *h, void *acc, int64_t nelem);
  * at the end (room for G + 1 entries); returns n, or a negative error.
  * wave_tiles <= 0: no batching. */
 int fo_overlap_plan_batches(const int32_t *cseg_host, int G, int wave_tiles, int32_t *first);
+/* The schedule of fo_overlap_gemm_allreduce_norm's normalisation (no counterpart in
+ * the reference): runs[3k .. 3k+2] = {batch, first tile row, end tile row} says that
+ * tile rows [first, end) of the output are normalised behind batch `batch` of
+ * fo_overlap_plan_batches(cseg_host, G, wave_tiles, ...), i.e. as soon as the groups
+ * holding all their tiles have been consumed.  At most four runs follow a batch that
+ * is not the last (what a scattered reorder table leaves over goes behind the last
+ * one).  RA_host: the reorder table [TM, TN] on the host.  Returns the number of
+ * runs, FO_ERR_LIMIT if there are more than max_runs, or a negative error. */
+int fo_overlap_plan_norm_rows(const int32_t *RA_host, int TM, int TN, const int32_t *cseg_host, int G,
+                              int wave_tiles, int32_t *runs, int max_runs);
 /* fused < 0 (default): chosen per call.  A GEMM below 6.4e10 flop (about 50 us)
  * keeps the whole call on the GEMM stream (the GEMM with its reordered store,
  * then one consumer launch: nothing that short can hide a fork and a join, and

@@ -320,6 +320,86 @@ def test_same_wave_groups_share_a_launch():
         plan([4, 0, 4], 8)
 
 
+def _norm_rows_restated(RA, cseg, wave_tiles, max_runs=4):
+    """The schedule of the normalisation, written down again from its description: behind every batch of
+    groups, the tile rows all of whose storage slots lie in groups consumed so far, as maximal runs of
+    consecutive rows in ascending order; a batch that is not the last takes at most max_runs runs."""
+    TM = RA.shape[0]
+    last = RA.max(axis=1)
+    emitted = np.zeros(TM, dtype=bool)
+    out, done = [], 0
+    batches = _capi.plan_batches(cseg, wave_tiles)
+    for b, (i, j) in enumerate(batches):
+        done += sum(cseg[i:j])
+        ready = [tm for tm in range(TM) if not emitted[tm] and last[tm] < done]
+        runs = []
+        for tm in ready:
+            if runs and runs[-1][1] == tm:
+                runs[-1][1] = tm + 1
+            else:
+                runs.append([tm, tm + 1])
+        if b < len(batches) - 1:
+            runs = runs[:max_runs]
+        for f, e in runs:
+            emitted[f:e] = True
+            out.append((b, f, e))
+    assert emitted.all()
+    return out
+
+
+def test_normalisation_follows_the_groups_that_complete_its_rows():
+    """fo_overlap_plan_norm_rows (the planner fo_overlap_gemm_allreduce_norm enqueues from) against a restatement,
+    on the large square's own tables, on scattered reorder tables and on random ones; every tile row is
+    normalised exactly once and never before the batch that holds its last tile."""
+    # the large square: 64 x 32 reorder tiles, 8 groups, waves of 512 tiles that cover 16 tile rows each
+    algo = _capi.find_algo(128, 256, swizzle=4)
+    M = N = 8192
+    TM, TN = M // 128, N // 256
+    hint = _capi.schedule_order(algo, M, N)
+    RA = layout.reorder_indices(TM * TN, hint, device="cpu").reshape(TM, TN).numpy()
+    cseg = [256] * 8
+    wave = 512
+    got = _capi.plan_norm_rows(RA, cseg, wave)
+    assert got == [(0, 0, 16), (1, 16, 32), (2, 32, 48), (3, 48, 64)]
+    assert got == _norm_rows_restated(RA, cseg, wave)
+    # identity table, groups that cut through tile rows: a row is ready with the group that holds its last tile
+    RA = np.arange(12, dtype=np.int32).reshape(4, 3)
+    assert _capi.plan_norm_rows(RA, [4, 4, 4], 0) == [(0, 0, 1), (1, 1, 2), (2, 2, 4)]
+    # every row has a tile in the last slot range: nothing before the last batch
+    RA = np.array([[0, 11], [1, 10], [2, 9], [3, 8], [4, 7], [5, 6]], dtype=np.int32)
+    assert _capi.plan_norm_rows(RA, [3, 3, 6], 0) == [(2, 0, 6)]
+    # alternate rows complete early: six single-row runs, of which a batch that is not the last takes four
+    RA = np.zeros((12, 2), dtype=np.int32)
+    RA[0::2] = np.arange(12).reshape(6, 2)
+    RA[1::2] = np.arange(12, 24).reshape(6, 2)
+    got = _capi.plan_norm_rows(RA, [12, 12], 0)
+    assert got == _norm_rows_restated(RA, [12, 12], 0)
+    assert [r for r in got if r[0] == 0] == [(0, 0, 1), (0, 2, 3), (0, 4, 5), (0, 6, 7)]
+    assert [r for r in got if r[0] == 1] == [(1, 1, 2), (1, 3, 4), (1, 5, 6), (1, 7, 12)]   # the last batch takes what is left
+    rng = np.random.default_rng(11)
+    for _ in range(60):
+        TM, TN = int(rng.integers(1, 9)), int(rng.integers(1, 6))
+        T = TM * TN
+        RA = rng.permutation(T).astype(np.int32).reshape(TM, TN)
+        if rng.random() < 0.5:            # tables that mostly follow the rows, as the schedule order does
+            RA = np.sort(RA.reshape(-1)).reshape(TM, TN)[rng.permutation(TM)]
+        cuts = sorted(rng.choice(np.arange(1, T), size=min(T - 1, int(rng.integers(0, 5))), replace=False).tolist()) if T > 1 else []
+        cseg = [b - a for a, b in zip([0] + cuts, cuts + [T])]
+        wave = int(rng.choice([0, 2, 5, T]))
+        got = _capi.plan_norm_rows(RA, cseg, wave)
+        assert got == _norm_rows_restated(RA, cseg, wave), (RA.tolist(), cseg, wave)
+        covered = np.zeros(TM, dtype=int)
+        ends = np.cumsum([sum(cseg[i:j]) for i, j in _capi.plan_batches(cseg, wave)])
+        for b, f, e in got:
+            covered[f:e] += 1
+            assert RA[f:e].max() < ends[b]
+        assert (covered == 1).all()
+    with pytest.raises(_capi.FlashOverlapError):
+        _capi.plan_norm_rows(np.array([[0, 5]], dtype=np.int32), [2], 0)      # an entry outside the table
+    with pytest.raises(_capi.FlashOverlapError):
+        _capi.plan_norm_rows(np.arange(4, dtype=np.int32).reshape(2, 2), [3], 0)  # groups do not cover the tiles
+
+
 def test_front_ends_refuse_undersized_buffers():
     """MM, RA, RE and D are indexed through raw pointers by kernels that store and count through them;
     both front ends must refuse buffers that are too small before anything is launched.  The case the
