@@ -826,7 +826,6 @@ __global__ void fo_pace_kernel(long long ticks) {
     const long long t0 = wall_clock64();
     while ((long long)wall_clock64() - t0 < ticks) __builtin_amdgcn_s_sleep(32);
 }
-constexpr double kMaxPaceSeconds = 1.0;
 }  // namespace
 
 int fo_pace_with(double seconds, fo_stream_t stream) {

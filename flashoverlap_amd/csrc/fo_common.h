@@ -156,6 +156,7 @@ int fo_wait_groups_with(int count, const int32_t *expect_dev, int32_t *counters,
                         fo_stream_t stream);
 // words[0..n) = value by a small kernel (no memset node under stream capture); word `skip` keeps its value.
 int fo_fill_words(int32_t *words, int n, int value, fo_stream_t stream, int skip = -1);
+constexpr double kMaxPaceSeconds = 1.0;                // longest stretch fo_pace_with accepts
 int fo_pace_with(double seconds, fo_stream_t stream);  // a one-lane kernel that holds the stream that long
 
 // Raster of whole-row waves (xcd_remap == 2).  The persistent launch holds R workgroups, R / 8 on each

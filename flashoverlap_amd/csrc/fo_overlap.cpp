@@ -120,6 +120,13 @@ int link_time(const fo_overlap *h, int64_t bytes, fo_stream_t stream) {
     return fo_pace_with((double)bytes / h->link_bytes_per_s, stream);
 }
 
+// Asked before a call enqueues anything: the largest stretch it could ask for (all of C) must be one that
+// fo_pace_with accepts, so that a refusal cannot come between the fork and the join.
+int link_fits(const fo_overlap *h, int64_t bytes) {
+    if (h->link_bytes_per_s <= 0) return FO_OK;
+    return (double)bytes / h->link_bytes_per_s > kMaxPaceSeconds ? FO_ERR_LIMIT : FO_OK;
+}
+
 int check_segments(const int32_t *cseg_host, int G, long tiles) {
     if (!cseg_host || G <= 0) return FO_ERR_SEGMENTS;
     long sum = 0;
@@ -384,6 +391,8 @@ int allreduce_overlap(fo_overlap *h, int dtype, int M, int N, int K, const void 
     if (rc) return rc;
     const int64_t tile_elems = (int64_t)info[0] * info[1];
     if (h->acc && h->acc_nelem < (int64_t)M * N) return FO_ERR_ARG;
+    rc = link_fits(h, (int64_t)M * N * 2);
+    if (rc) return rc;
     std::vector<long> last_slot;  // per tile row: its largest storage slot
     if (np) {
         if (!np->Y || !np->Wt || !np->RA_host) return FO_ERR_ARG;
@@ -543,6 +552,8 @@ extern "C" int fo_overlap_gemm_reducescatter(fo_overlap_t *h, int dtype, int M, 
     if (tile_elems % (8 * W) || ((int64_t)M * N) % W) return FO_ERR_SHAPE;
     const int64_t seg_stride = (int64_t)M * N / W;
     if (h->acc && h->acc_nelem < (int64_t)M * N) return FO_ERR_ARG;
+    rc = link_fits(h, (int64_t)M * N * 2);
+    if (rc) return rc;
 
     const bool same_stream = in_stream(h, M, N, K);
     const int fused = same_stream ? 0 : fused_grid(h, G);

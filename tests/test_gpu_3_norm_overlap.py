@@ -265,5 +265,12 @@ def test_link_rate_model_holds_the_consumer_stream_and_changes_no_result(fo):
         fo.ops.pace(2_000_000_000)
     with pytest.raises(RuntimeError):
         ov.set_link_rate(-1.0)
+    # a rate that would hold the stream for more than a second is refused before anything is enqueued
+    ov.set_link_rate(0.001)
+    MM.zero_()
+    with pytest.raises(RuntimeError):
+        ov.gemm_allreduce_rmsnorm_overlap(A, B, C, MM, RA, RA_cpu, 1, cs_cpu, cs_gpu, algo, Y, gamma, eps=EPS)
+    torch.cuda.synchronize()
+    assert ov.status() == 0 and (MM == 0).all()
     ov.set_link_rate(0)
     ov.close()
