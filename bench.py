@@ -337,8 +337,10 @@ def measure(args, workload, compact=False):
     def vendor_gemm():
         torch.matmul(A, B.t(), out=Cplain)
     ms_vendor, _ = timed(vendor_gemm, K_, W_)
-    ms_consumer, _ = timed(consumer_alone, K_, W_)
-    ms_norm, _ = timed(norm, K_, W_)
+    # the two bandwidth-bound kernels last tens of microseconds: 200 launches or more per figure, so that the
+    # first launch's start-up (several microseconds after a synchronisation) does not weigh on the average
+    ms_consumer, _ = timed(consumer_alone, max(200, K_), W_)
+    ms_norm, _ = timed(norm, max(200, K_), W_)
     ACC.zero_()
     torch.cuda.synchronize()
 
